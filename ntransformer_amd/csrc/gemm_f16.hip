@@ -896,7 +896,6 @@ __global__ __launch_bounds__(256, GB_WG_PER_CU) void gemm_quant_f16_kernel(const
     // The ring's loads and the stores that consume them are inline asm: a load the compiler tracks makes it wait, at the consumer, for
     // "all but the tracked loads younger than it" -- it does not see the LDS-DMA requests in between, so that wait drained the whole
     // activation ring at every unit boundary (round 3, the ISA of the first deep-ring build).  Here every wait is explicit and exact.
-    // (The ring registers appear in no compiler-generated instruction: tools/check_gemm_isa.py checks the build for that.)
     u32x4 ring[NRING][NLD];
     auto load_unit = [&](int k, int urel) {   // unit `urel` of this split (past the end: the last one again, multiplied by zeros)
         if (kGbAblate & 32) { if (urel >= 2) return; }
