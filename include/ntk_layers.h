@@ -1,5 +1,5 @@
-/* include/ntk_layers.h -- operators of the layer-list model families (csrc/dense.hip, csrc/latent_attention.hip, csrc/moe.hip,
- * csrc/layer_ops.hip): dense bfloat16 / float32 weights, F32 activations and residual stream.
+/* include/ntk_layers.h -- operators of the layer-list model families (csrc/dense.hip, csrc/latent_attention.hip, csrc/window_attention.hip,
+ * csrc/lightning_attention.hip, csrc/gated_recurrence.hip, csrc/moe.hip, csrc/layer_ops.hip): dense bfloat16 / float32 weights, F32 activations and residual stream.
  *
  * Same conventions as ntk.h: plain pointers and sizes, stream ordered, no allocation, NTK_OK or a negative NTK_E_* code.  Nothing here knows a
  * model: every size and constant is a parameter.  Two precisions of one operator set:
@@ -43,6 +43,9 @@ typedef struct ntk_dense_desc {
     /* what is added to the (clamped) up value inside the gated activation: 1 for the clipped form above, 0 for a plain gated unit
      * (g * sigmoid(alpha * g) * u; glu_limit = INFINITY switches the clamps off: silu(g) * u with alpha 1) */
     float glu_up_offset;
+    /* a cubic term inside the gate's sigmoid: act(g') = g' * sigmoid(glu_alpha * (g' + glu_cubic * g'^3)).  0: none.  alpha = 2 sqrt(2 / pi) and
+     * cubic = 0.044715 give the tanh form of gelu, 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3))), since 0.5 (1 + tanh y) = sigmoid(2 y) */
+    float glu_cubic;
 } ntk_dense_desc;
 int ntk_dense_few_rows(void);   /* up to this many rows a product takes the row-streaming form */
 int ntk_dense(const ntk_dense_desc* d, void* stream);
@@ -93,6 +96,36 @@ int ntk_polynorm(float* y, int ldy, const float* z, int ldz, const float* coef, 
 /* y[t][i] = x[t][i] / sqrt(mean(x[t]^2) + eps) * w[i] * sigmoid(g[t][i]) (the norm runs over the whole row of n values; g rows ldg apart, g may be NULL) */
 int ntk_gated_rmsnorm(float* y, int ldy, const float* x, int ldx, const float* w, const float* g, int ldg, int T, int n, float eps, void* stream);
 
+/* Dynamic-tanh norm (no mean, no variance): y[t][i] = tanh(alpha * x[t][i]) * w[i] + b[i], alpha one number per norm; b may be NULL */
+int ntk_dyt(float* y, int ldy, const float* x, int ldx, const float* w, const float* b, float alpha, int T, int n, void* stream);
+/* out[t][:] = table[tokens[t]][:] + pos_table[pos0 + t][:] (both NTK_DT_BF16 or both NTK_DT_F32, the sum in F32; a learned vector per position, n_pos rows),
+ * then, if w: the dynamic-tanh norm above with (w, b, alpha).  copy (may be NULL) receives the same rows. */
+int ntk_embed_positions(float* out, float* copy, const void* table, const void* pos_table, int tdtype, const int* tokens, int T, int vocab, int width, int pos0,
+                        int n_pos, const float* w, const float* b, float alpha, void* stream);
+/* y[t][i] = y[t][i] * sigmoid(g[t][i] + (gb ? gb[i] : 0)) * scale */
+int ntk_sigmoid_gate_scaled(float* y, int ldy, const float* g, int ldg, const float* gb, float scale, int T, int n, void* stream);
+/* x[t][i] = tanh(x[t][i]) over T rows of n */
+int ntk_tanh_rows(float* x, int ldx, int T, int n, void* stream);
+/* Per head: y[t][h][c] = x[t][h][c] / sqrt(mean_c(x[t][h]^2) + eps) * w[h * w_head_stride + c] * act(g[t][h][c]) * scale, the mean over the head's dv values.
+ * w_head_stride 0: one weight vector [dv] shared by the heads; dv: a weight per head and column.  act 0: no gate (g unused), 1: sigmoid, 2: silu. */
+int ntk_head_rmsnorm_gate(float* y, int ldy, const float* x, int ldx, const float* w, int w_head_stride, const float* g, int ldg, int act, float scale, int T, int H,
+                          int dv, float eps, void* stream);
+/* The seam of a layer whose sublayer results join the stream through a gate and whose layer results are averaged over depth, in one launch:
+ *   r[t]  = x[t] + (y[t] + yb) * sigmoid(g[t] + gb)                (yb, gb: bias vectors [n], may be NULL)
+ *   n_hist == 0:  x[t] = r[t]
+ *   n_hist  > 0:  hist[n_hist - 1][t] = r[t];  x[t] = sum_{j < n_hist} coef[j] * hist[j][t]   (j ascending, F32; hist entries hist_stride floats apart, rows of n;
+ *                 coef device F32 [n_hist])
+ *   h != NULL:    h[t] = tanh(alpha * x[t]) * nw + nb               (the dynamic-tanh norm in front of the next sublayer)                              */
+typedef struct ntk_gated_seam_desc {
+    float* x; int ldx;
+    const float* y; int ldy; const float* yb;
+    const float* g; int ldg; const float* gb;
+    float* hist; long long hist_stride; int n_hist; const float* coef;
+    float* h; int ldh; const float* nw; const float* nb; float alpha;
+    int T, n;
+} ntk_gated_seam_desc;
+int ntk_gated_seam(const ntk_gated_seam_desc* d, void* stream);
+
 /* ---- latent_attention.hip ---------------------------------------------------------------------------------------------------------
  * Attention whose keys and values are up-projections of one cached latent per position plus one rotated key part shared by the heads.
  * The cache of a layer run holds rows of `row` = kv_rank + rot_dim floats: [latent (normed) | rotated key part].                       */
@@ -132,6 +165,12 @@ int ntk_latent_unfold_value(float* out, int ldo, const float* lat, const void* w
  * (2i, 2i+1) paired; the rest unchanged) and copies v behind the keys. */
 int ntk_window_prepare(float* cache, int row, float* q, int ldq, const float* k, int ldk, const float* v, int ldv, int H, int G, int maps, int dn, int dv,
                        const ntk_rotary* rot, int pos0, int T, void* stream);
+/* The same with what a projection leaves to its consumer: q = (q + qb) * (1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)) at position p before the
+ * rotation (a query temperature that grows with the position; temp_coef 0: none), k + kb and v + vb into the cache rows.  qb [H*maps*dn], kb [G*maps*dn],
+ * vb [G*dv] device F32, each may be NULL.  rot->dims may be 0 (no rotation). */
+int ntk_window_prepare_biased(float* cache, int row, float* q, int ldq, const float* k, int ldk, const float* v, int ldv, int H, int G, int maps, int dn, int dv,
+                              const ntk_rotary* rot, const float* qb, const float* kb, const float* vb, float temp_coef, double temp_every, int pos0, int T,
+                              void* stream);
 /* a_m = softmax_j(scale * q_m . k_m[j]) V over the visible j (j <= p, and p - j < window if window > 0), per map m.
  * maps == 1: out = a_0.  maps == 2: out = a_0 - lambda * a_1 (a differential pair).  sub_norm != 0: out is then divided by sqrt(mean(out^2) + eps) over
  * the head's dv values.  out_scale multiplies the result.  out [T][H][dv], ldo floats between tokens.
@@ -145,6 +184,9 @@ typedef struct ntk_window_attention_desc {
     float scale, lambda;
     int sub_norm; float eps, out_scale;
     float* scratch;
+    /* a learned bias by distance, added to the scaled score (not scaled itself): rel[bucket_of[min(p - j, n_dist - 1)] * H + h].
+     * rel device F32 [buckets][H], bucket_of device int [n_dist].  rel == NULL: none. */
+    const float* rel; const int* bucket_of; int n_dist;
 } ntk_window_attention_desc;
 size_t ntk_window_attention_scratch(int T, int H, int maps, int dv, int nkeys);
 int ntk_window_attention(const ntk_window_attention_desc* d, void* stream);
@@ -159,6 +201,34 @@ int ntk_window_attention(const ntk_window_attention_desc* d, void* stream);
 size_t ntk_lightning_attention_scratch(int T, int H, int dn, int dv);
 int ntk_lightning_attention(float* out, int ldo, const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* log_decay, float* state,
                             int H, int dn, int dv, int silu, int pos0, int T, float* scratch, void* stream);
+
+/* ---- gated_recurrence.hip -----------------------------------------------------------------------------------------------------------
+ * Linear attention whose state forgets per token, head and KEY CHANNEL, optionally with the delta rule's removal term (taken from S_(t-1) as it was):
+ *     S_t = diag(w_t) S_(t-1) - (a_t * u_t) (u_t^T S_(t-1)) + k_t v_t^T,      o_t = S_t^T (q_scale * q_t),      u_t = k_t / sqrt(sum(k_t^2) + unit_eps)
+ * S [dn][dv] per head, F32; everything after the projections is F32.  q, k, wz [T][H][dn], v [T][H][dv] (ld* floats between tokens).
+ * The decay comes from the raw projection wz (+ wb [H*dn], may be NULL) by `decay_form`:
+ *     NTK_DECAY_SIGMOID_ROOT   w = sigmoid(z)^(1 / decay_param)            (formed as exp(log sigmoid(z) / param))
+ *     NTK_DECAY_EXP_SIGMOID    w = exp(-decay_param * sigmoid(z))
+ *     NTK_DECAY_GIVEN          w = z
+ * az (may be NULL: no removal term -- gated linear attention): a = sigmoid(az + ab), [T][H][dn] (+ ab [H*dn], may be NULL).
+ * state [H][dn][dv]: read unless pos0 == 0 (a sequence starts from zeros), written at the end.  out [T][H][dv].  dn <= 1024.
+ * A lane owns a few state rows of one column; tokens are walked in order, so a portion cut anywhere gives the same sums in the same order. */
+#define NTK_DECAY_GIVEN 0
+#define NTK_DECAY_SIGMOID_ROOT 1
+#define NTK_DECAY_EXP_SIGMOID 2
+typedef struct ntk_gated_recurrence_desc {
+    float* out; int ldo;
+    const float* q; int ldq;
+    const float* k; int ldk;
+    const float* v; int ldv;
+    const float* wz; int ldw; const float* wb; int decay_form; float decay_param;
+    const float* az; int lda; const float* ab; float unit_eps;
+    float* state;
+    int H, dn, dv;
+    float q_scale;
+    int pos0, T;
+} ntk_gated_recurrence_desc;
+int ntk_gated_recurrence(const ntk_gated_recurrence_desc* d, void* stream);
 
 /* ---- moe.hip ---------------------------------------------------------------------------------------------------------------------- */
 /* Router of a mixture of experts, one launch: z = W_r h (F32 weights [E][n]), s = softmax(z); the `top` largest (ties: the lower index), weights
@@ -183,6 +253,9 @@ int ntk_moe_group(int* offsets, int* order, int* where, const int* ids, int T, i
 int ntk_clipped_glu(float* a, const float* gu, int rows, int ff, float limit, float alpha, void* stream);
 /* the general gated unit: a[r][f] = g' * sigmoid(alpha * g') * (u' + up_offset) with the clamps of ntk_clipped_glu (limit = INFINITY: none) */
 int ntk_glu(float* a, const float* gu, int rows, int ff, float limit, float alpha, float up_offset, void* stream);
+/* ... with a cubic term inside the sigmoid, g' * sigmoid(alpha * (g' + cubic * g'^3)) * (u' + up_offset) (the tanh form of gelu: see ntk_dense_desc), and gu rows
+ * ldgu floats apart (gate values at [0, ff), up values at [ff, 2 ff)) */
+int ntk_glu_cubic(float* a, const float* gu, int ldgu, int rows, int ff, float limit, float alpha, float cubic, float up_offset, void* stream);
 /* out[t][:] = sum_s wts[t][s] * d[where[t*top+s]][:] + (sgate ? sgate[t] : 1) * shared[t][:] (if shared): the experts' sum on its own, for layers that norm it before
  * it joins the stream */
 int ntk_moe_sum(float* out, const float* d, const int* where, const float* wts, const float* shared, const float* sgate, int T, int top, int n, void* stream);

@@ -32,7 +32,7 @@ struct DenseArgs {
     const int* offsets;
     const int* rows; int row_div;
     int T, N, K, accumulate, G, vec;
-    int glu_ff; float glu_limit, glu_alpha, glu_up_offset;   // few-row form only: outputs f < glu_ff = gated unit of rows f (gate) and glu_ff + f (up)
+    int glu_ff; float glu_limit, glu_alpha, glu_up_offset, glu_cubic;   // few-row form only: outputs f < glu_ff = gated unit of rows f (gate) and glu_ff + f (up)
     const float* norm_w; float norm_eps, norm_offset;   // few-row form only: the activation row is RMS-normed with weight (offset + norm_w) first
 };
 
@@ -304,7 +304,8 @@ __global__ __launch_bounds__(256) void dense_gemv_kernel(const DenseArgs a) {
             float t = s[i];
             if constexpr (GLU) {
                 const float gg = fminf(s[i], a.glu_limit), uu = fminf(fmaxf(s[i + OUT], -a.glu_limit), a.glu_limit);
-                t = gg * (1.0f / (1.0f + expf(-a.glu_alpha * gg))) * (uu + a.glu_up_offset);
+                const float zz = a.glu_cubic != 0.0f ? fmaf(a.glu_cubic * gg * gg, gg, gg) : gg;
+                t = gg * (1.0f / (1.0f + expf(-a.glu_alpha * zz))) * (uu + a.glu_up_offset);
             }
             float* y = a.Y + (long long)r * a.ldy + n0 + i;
             *y = a.accumulate ? *y + t : t;
@@ -350,11 +351,11 @@ int ntk_dense(const ntk_dense_desc* d, void* stream) {
     if (d->norm_w && d->T > kGemvRows) return NTK_E_SHAPE;
     if (d->T == 0) return NTK_OK;
     const int G = d->offsets ? d->G : 1;
-    DenseArgs a{d->Y, d->ldy, d->X, d->ldx, d->W, d->wstride, d->offsets, d->rows, d->rows ? d->row_div : 1, d->T, d->N, d->K, d->accumulate, G, 0, 0, 0.0f, 0.0f, 0.0f, nullptr, 0.0f, 0.0f};
+    DenseArgs a{d->Y, d->ldy, d->X, d->ldx, d->W, d->wstride, d->offsets, d->rows, d->rows ? d->row_div : 1, d->T, d->N, d->K, d->accumulate, G, 0, 0, 0.0f, 0.0f, 0.0f, 0.0f, nullptr, 0.0f, 0.0f};
     hipStream_t s = resolve_stream(stream);
     if (d->T <= kGemvRows) {
         if ((size_t)d->K * 4 > 160 * 1024 - 1024) return NTK_E_SHAPE;
-        a.glu_ff = d->glu_ff; a.glu_limit = d->glu_limit; a.glu_alpha = d->glu_alpha; a.glu_up_offset = d->glu_up_offset;
+        a.glu_ff = d->glu_ff; a.glu_limit = d->glu_limit; a.glu_alpha = d->glu_alpha; a.glu_up_offset = d->glu_up_offset; a.glu_cubic = d->glu_cubic;
         a.norm_w = d->norm_w; a.norm_eps = d->norm_eps; a.norm_offset = d->norm_offset;
         a.vec = (d->K % 8 == 0) && !((uintptr_t)d->W & 15) && !((d->wstride * (d->wdtype == NTK_DT_BF16 ? 2 : 4)) & 15);
         if (d->wdtype == NTK_DT_BF16) launch_gemv<uint16_t>(a, d->T, s);

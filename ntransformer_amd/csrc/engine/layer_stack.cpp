@@ -20,6 +20,17 @@ static StackForm sequential_form() {
     f.sequential = true; f.loop_projection = false; f.router_score = 1; f.router_renorm = false; f.clipped_glu = false; f.shared_gate = false; f.group_top = 2;
     return f;
 }
+static StackForm gated_form() {
+    StackForm f;
+    f.gated = true; f.loop_projection = false;
+    return f;
+}
+// what the gated form's mechanisms fix
+static constexpr float kGeluAlpha = 1.5957691216057308f;   // 2 sqrt(2 / pi): 0.5 (1 + tanh y) = sigmoid(2 y)
+static constexpr float kGeluCubic = 0.044715f;
+static constexpr float kDeltaDecayRate = 0.6065306597126334f;   // exp(-1/2): w = exp(-rate * sigmoid(.))
+static constexpr float kUnitKeyEps = 1e-6f;
+static FamilyRegistrar reg_tubazen("Tubazen", [] { return std::unique_ptr<SequenceModel>(new LayerStackModel(gated_form())); });
 static FamilyRegistrar reg_fabolorn("Fabolorn", [] { return std::unique_ptr<SequenceModel>(new LayerStackModel(parallel_form())); });
 static FamilyRegistrar reg_nizorax("Nizorax", [] { return std::unique_ptr<SequenceModel>(new LayerStackModel(sequential_form())); });
 
@@ -161,13 +172,54 @@ int LayerStackModel::parse_lightning(const Json& L, LightningMixer& m) {
     return NTK_OK;
 }
 
+int LayerStackModel::parse_gla(const Json& L, GlaMixer& m) {
+    const Json& mx = L.at("mixer");
+    const std::string where = "mixer 'gla'";
+    if (!mx.is_object()) return fail(NTK_E_FORMAT, where + ": no 'mixer' object");
+    if (!need_int(mx, "heads", m.heads, err_, where) || !need_int(mx, "dim", m.dim, err_, where) || !need_int(mx, "vdim", m.vdim, err_, where)) return NTK_E_FORMAT;
+    if (!mx.at("tau").is_number() || !(mx.at("tau").number() > 0.0)) return fail(NTK_E_FORMAT, where + ": 'tau' must be a positive number");
+    m.tau = (float)mx.at("tau").number();
+    if (m.dim > 1024 || m.vdim > 1024) return fail(NTK_E_SHAPE, where + ": dim and vdim up to 1024 are supported");
+    return NTK_OK;
+}
+
+int LayerStackModel::parse_parallel(const Json& L, ParallelMixer& m) {
+    const Json& mx = L.at("mixer");
+    const std::string where = "mixer 'parallel'";
+    if (!mx.is_object() || !mx.at("left").is_object() || !mx.at("right").is_object()) return fail(NTK_E_FORMAT, where + ": 'mixer' needs 'left' and 'right'");
+    const Json& l = mx.at("left");
+    const Json& r = mx.at("right");
+    BiasedAttention& a = m.left;
+    if (!need_int(l, "heads", a.heads, err_, where + " left") || !need_int(l, "dim", a.dim, err_, where + " left") || !need_int(l, "vdim", a.vdim, err_, where + " left")) return NTK_E_FORMAT;
+    a.kv_heads = a.heads;
+    if (l.has("kv_heads") && !need_int(l, "kv_heads", a.kv_heads, err_, where + " left")) return NTK_E_FORMAT;
+    if (a.heads % a.kv_heads) return fail(NTK_E_FORMAT, where + ": heads must be a multiple of kv_heads");
+    if (!l.at("scale").is_number()) return fail(NTK_E_FORMAT, where + ": 'scale' is missing");
+    a.scale = (float)l.at("scale").number();
+    if (!l.at("bias_max").is_number() || !(l.at("bias_max").number() > 0.0)) return fail(NTK_E_FORMAT, where + ": 'bias_max' is missing");
+    a.bias_max = l.at("bias_max").number();
+    a.temp_coef = 0.0f; a.temp_every = 1.0;
+    if (l.has("q_temp")) {
+        a.temp_coef = (float)l.at("q_temp").at("coef").number(0.0);
+        a.temp_every = l.at("q_temp").at("every").number(1.0);
+        if (!(a.temp_every > 0.0)) return fail(NTK_E_FORMAT, where + ": q_temp.every must be positive");
+    }
+    if (a.vdim > 512) return fail(NTK_E_SHAPE, where + ": vdim up to 512 is supported");
+    if (!need_int(r, "heads", m.right.heads, err_, where + " right") || !need_int(r, "dim", m.right.dim, err_, where + " right")) return NTK_E_FORMAT;
+    if (m.right.dim > 1024) return fail(NTK_E_SHAPE, where + ": dim up to 1024 is supported");
+    m.left_scale = (float)mx.at("left_scale").number(1.0);
+    m.right_scale = (float)mx.at("right_scale").number(1.0);
+    return NTK_OK;
+}
+
 int LayerStackModel::parse_mlp(const Json& ml, const std::string& where, StackLayer& S) {
     const std::string kind = ml.at("kind").is_string() ? ml.at("kind").str : "moe";
     if (kind == "dense") {
         S.mlp_kind = kMlpDense;
-        if (!need_int(ml, "ff", S.ffn.ff, err_, where)) return NTK_E_FORMAT;
+        if (!need_int(ml, "ff", form_.gated ? S.gff.ff : S.ffn.ff, err_, where)) return NTK_E_FORMAT;
         return NTK_OK;
     }
+    if (form_.gated) return fail(NTK_E_FORMAT, where + ": this family has the dense feed-forward only");
     if (kind != "moe") return fail(NTK_E_FORMAT, where + ": unknown kind '" + kind + "'");
     S.mlp_kind = kMlpMoe;
     MoeFeedForward& M = S.mlp;
@@ -206,6 +258,10 @@ int LayerStackModel::parse(const ModelFolder& f) {
         logit_scale_ = (float)c.at("logit_scale").number(1.0);
         has_state_ = taps_ > 1;
     }
+    if (form_.gated) {
+        logit_scale_ = (float)c.at("logit_scale").number(1.0);
+        has_state_ = true;
+    }
     if (c.at("bos").is_number()) info_.bos = (int)c.at("bos").integer();
     if (c.at("eos").is_number()) info_.eos = (int)c.at("eos").integer();
     const Json& ls = c.at("layers");
@@ -216,18 +272,21 @@ int LayerStackModel::parse(const ModelFolder& f) {
         StackLayer& S = layers_[i];
         S.type = L.at("type").str;
         // which mixers a form lists: the parallel form's layers read two norms of one input, so its mixers are the latent kinds it was built around
-        if (!form_.sequential && (S.type == "latent_attention" || S.type == "latent_attention_2")) { S.mixer = kMixLatent; LS_TRY(parse_mixer(L, S.type, S.mix)); }
+        if (form_.gated && S.type == "gla") { S.mixer = kMixGla; LS_TRY(parse_gla(L, S.gla)); }
+        else if (form_.gated && S.type == "parallel") { S.mixer = kMixParallel; LS_TRY(parse_parallel(L, S.par)); }
+        else if (form_.gated) return fail(NTK_E_FORMAT, "layer " + std::to_string(i) + ": unknown mixer type '" + S.type + "'");
+        else if (!form_.sequential && (S.type == "latent_attention" || S.type == "latent_attention_2")) { S.mixer = kMixLatent; LS_TRY(parse_mixer(L, S.type, S.mix)); }
         else if (form_.sequential && S.type == "attention") { S.mixer = kMixWindow; LS_TRY(parse_window(L, S.att)); }
         else if (form_.sequential && S.type == "lightning") { S.mixer = kMixLightning; LS_TRY(parse_lightning(L, S.lin)); has_state_ = true; }
         else return fail(NTK_E_FORMAT, "layer " + std::to_string(i) + ": unknown mixer type '" + S.type + "'");
-        S.has_mlp = L.has("mlp");
+        S.has_mlp = L.has("mlp") && !L.at("mlp").is_null();
         if (S.has_mlp) LS_TRY(parse_mlp(L.at("mlp"), "layer " + std::to_string(i) + " mlp", S));
-        if (!form_.sequential && S.mlp_kind == kMlpDense) return fail(NTK_E_FORMAT, "layer " + std::to_string(i) + ": this family has no dense feed-forward");
+        if (!form_.sequential && !form_.gated && S.mlp_kind == kMlpDense) return fail(NTK_E_FORMAT, "layer " + std::to_string(i) + ": this family has no dense feed-forward");
     }
     // the order of layer runs
     const int n = (int)layers_.size();
     runs_.clear();
-    has_loop_ = c.has("loop");
+    has_loop_ = c.has("loop") && !form_.gated;   // (the gated form's depth weights are per layer: it has no repeated span)
     if (has_loop_) {
         const Json& lp = c.at("loop");
         const int a = (int)lp.at("start").integer(), b = (int)lp.at("stop").integer(), times = (int)lp.at("times").integer(1);
@@ -309,9 +368,128 @@ int LayerStackModel::upload_matrix(const ModelFolder& f, const std::vector<std::
     return NTK_OK;
 }
 
+int LayerStackModel::read_scalar(const ModelFolder& f, const std::string& name, float* out) {
+    const StTensor* t = f.tensor(name);
+    if (!t) return fail(NTK_E_FORMAT, "tensor '" + name + "' is missing");
+    if (t->numel() != 1) return fail(NTK_E_SHAPE, "tensor '" + name + "' is not one number");
+    if (!tensor_to_f32(*t, out)) return fail(NTK_E_DTYPE, "tensor '" + name + "': dtype " + t->dtype + " is not supported");
+    weight_bytes_ += t->nbytes;
+    return NTK_OK;
+}
+
+// matrices with the same number of rows side by side: row r of the result = [row r of the first | row r of the second | ...]
+int LayerStackModel::upload_hstack(const ModelFolder& f, const std::vector<std::string>& names, DenseW& out) {
+    int64_t rows = -1, cols = 0;
+    for (const auto& nm : names) {
+        const StTensor* t = f.tensor(nm);
+        if (!t) return fail(NTK_E_FORMAT, "tensor '" + nm + "' is missing");
+        if (t->shape.size() != 2 || (rows >= 0 && t->shape[0] != rows)) return fail(NTK_E_SHAPE, "tensor '" + nm + "': expected a matrix with the rows of its neighbours");
+        rows = t->shape[0];
+        cols += t->shape[1];
+    }
+    const size_t es = wdtype_ == NTK_DT_BF16 ? 2 : 4;
+    std::vector<uint8_t> h((size_t)rows * cols * es);
+    int64_t c0 = 0;
+    for (const auto& nm : names) {
+        const StTensor* t = f.tensor(nm);
+        const int64_t n = t->shape[1];
+        std::vector<float> tmp((size_t)t->numel());
+        if (!tensor_to_f32(*t, tmp.data())) return fail(NTK_E_DTYPE, "tensor '" + nm + "': dtype " + t->dtype + " is not supported");
+        for (int64_t r = 0; r < rows; ++r)
+            for (int64_t c = 0; c < n; ++c) {
+                const float v = tmp[(size_t)(r * n + c)];
+                if (wdtype_ == NTK_DT_BF16) ((uint16_t*)h.data())[r * cols + c0 + c] = f32_to_bf16(v);   // (exact for values that were bfloat16)
+                else ((float*)h.data())[r * cols + c0 + c] = v;
+            }
+        c0 += n;
+        weight_bytes_ += t->nbytes;
+    }
+    out.ptr = dev_alloc(h.size() + 256);
+    if (!out.ptr) return fail(NTK_E_NOMEM, "out of device memory");
+    nt_hip_memcpy_h2d(out.ptr, h.data(), h.size());
+    out.dtype = wdtype_; out.in_f = cols; out.out_f = rows; out.count = 1;
+    return NTK_OK;
+}
+
 int LayerStackModel::upload_norm(const ModelFolder& f, const std::string& name, NormW& out) {
     LS_TRY(upload_vector(f, name, info_.width, &out.w));
-    if (form_.sequential) LS_TRY(upload_vector(f, name + ".b", info_.width, &out.b));
+    if (form_.sequential || form_.gated) LS_TRY(upload_vector(f, name + ".b", info_.width, &out.b));
+    if (form_.gated) LS_TRY(read_scalar(f, name + ".alpha", &out.alpha));
+    return NTK_OK;
+}
+
+// bucket of a distance n >= 0 for a table of B rows reaching out to distance D: the first B/2 distances have a row each, the rest share the other
+// rows on a logarithmic scale, everything from D on the last row.  Formed in F32 like every position quantity.
+static int distance_bucket(int n, int B, double D) {
+    const int half = B / 2;
+    if (n < half) return n;
+    const float num = std::log((float)n / (float)half), den = (float)std::log(D / (double)half);
+    const float v = num / den * (float)(B - half);
+    const long long b = (long long)half + (long long)std::floor(v);
+    return (int)std::min<long long>((long long)B - 1, std::max<long long>(b, 0));
+}
+
+int LayerStackModel::upload_gated_mixer(const ModelFolder& f, const std::string& p, int i, StackLayer& L) {
+    const int W = info_.width;
+    const std::string li = "layer " + std::to_string(i);
+    auto rows_of = [&](const std::string& nm) -> int64_t { const StTensor* t = f.tensor(nm); return t && t->shape.size() == 2 ? t->shape[0] : -1; };
+    if (L.mixer == kMixGla) {
+        GlaMixer& m = L.gla;
+        const int hq = m.heads * m.dim, hv = m.heads * m.vdim;
+        const int64_t rank = rows_of(p + "mix.a1");
+        if (rank <= 0) return fail(NTK_E_FORMAT, "tensor '" + p + "mix.a1' is missing");
+        m.rank = (int)rank;
+        LS_TRY(upload_matrix(f, {p + "mix.q", p + "mix.k", p + "mix.v", p + "mix.g", p + "mix.a1", p + "rg1"}, W, m.in));
+        m.k_off = hq; m.v_off = 2 * hq; m.g_off = 2 * hq + hv; m.a_off = 2 * hq + 2 * hv; m.rg_off = m.a_off + m.rank;
+        if (rows_of(p + "mix.q") != hq || rows_of(p + "mix.k") != hq || rows_of(p + "mix.v") != hv || rows_of(p + "mix.g") != hv || rows_of(p + "rg1") != W)
+            return fail(NTK_E_SHAPE, li + ": the mixer's input projections do not have the configured sizes");
+        LS_TRY(upload_matrix(f, {p + "mix.a2"}, m.rank, m.a2));
+        if (m.a2.out_f != hq) return fail(NTK_E_SHAPE, "tensor '" + p + "mix.a2' does not have heads * dim rows");
+        LS_TRY(upload_vector(f, p + "mix.a2.b", hq, &m.a2_b));
+        LS_TRY(upload_vector(f, p + "mix.norm", m.vdim, &m.norm));
+        LS_TRY(upload_matrix(f, {p + "mix.o"}, hv, m.o));
+        if (m.o.out_f != W) return fail(NTK_E_SHAPE, "tensor '" + p + "mix.o' does not have 'width' rows");
+        return NTK_OK;
+    }
+    ParallelMixer& m = L.par;
+    BiasedAttention& a = m.left;
+    DeltaMixer& d = m.right;
+    const std::string l = p + "mix.left.", r = p + "mix.right.";
+    const int hq = a.heads * a.dim, gk = a.kv_heads * a.dim, gv = a.kv_heads * a.vdim, hv = a.heads * a.vdim, hd = d.heads * d.dim;
+    const int64_t rank = rows_of(r + "w1");
+    if (rank <= 0) return fail(NTK_E_FORMAT, "tensor '" + r + "w1' is missing");
+    d.rank = (int)rank;
+    LS_TRY(upload_matrix(f, {l + "q", l + "k", l + "v", l + "g", r + "r", r + "k", r + "v", r + "g", r + "a", r + "w1", p + "rg1"}, W, m.in));
+    a.q_off = 0; a.k_off = hq; a.v_off = hq + gk; a.g_off = hq + gk + gv;
+    d.r_off = a.g_off + hv; d.k_off = d.r_off + hd; d.v_off = d.k_off + hd; d.g_off = d.v_off + hd; d.a_off = d.g_off + hd; d.w1_off = d.a_off + hd;
+    m.rg_off = d.w1_off + d.rank;
+    if (rows_of(l + "q") != hq || rows_of(l + "k") != gk || rows_of(l + "v") != gv || rows_of(l + "g") != hv || rows_of(r + "r") != hd || rows_of(r + "k") != hd ||
+        rows_of(r + "v") != hd || rows_of(r + "g") != hd || rows_of(r + "a") != hd || rows_of(p + "rg1") != W)
+        return fail(NTK_E_SHAPE, li + ": the mixer's input projections do not have the configured sizes");
+    LS_TRY(upload_vector(f, l + "q.b", hq, &a.q_b));
+    LS_TRY(upload_vector(f, l + "k.b", gk, &a.k_b));
+    LS_TRY(upload_vector(f, l + "v.b", gv, &a.v_b));
+    const StTensor* rel = f.tensor(l + "rel");
+    if (!rel || rel->shape.size() != 2 || rel->shape[1] != a.heads || rel->shape[0] < 2) return fail(NTK_E_SHAPE, "tensor '" + l + "rel' is not [buckets >= 2, heads]");
+    a.buckets = (int)rel->shape[0];
+    if (!(a.bias_max > a.buckets / 2)) return fail(NTK_E_FORMAT, li + ": bias_max must lie beyond the table's first half");
+    LS_TRY(upload_vector(f, l + "rel", (int64_t)a.buckets * a.heads, &a.rel));
+    {
+        std::vector<int> b((size_t)opt_.max_context);
+        for (int n = 0; n < opt_.max_context; ++n) b[(size_t)n] = distance_bucket(n, a.buckets, a.bias_max);
+        a.bucket_of = (int*)dev_alloc(b.size() * sizeof(int));
+        if (!a.bucket_of) return fail(NTK_E_NOMEM, "out of device memory");
+        nt_hip_memcpy_h2d(a.bucket_of, b.data(), b.size() * sizeof(int));
+    }
+    LS_TRY(upload_matrix(f, {r + "w2"}, d.rank, d.w2));
+    if (d.w2.out_f != hd) return fail(NTK_E_SHAPE, "tensor '" + r + "w2' does not have heads * dim rows");
+    LS_TRY(upload_vector(f, r + "w0", hd, &d.w0));
+    LS_TRY(upload_vector(f, r + "a.b", hd, &d.a_b));
+    LS_TRY(upload_vector(f, r + "norm", hd, &d.norm));
+    LS_TRY(upload_hstack(f, {l + "o", r + "o"}, m.o));
+    if (m.o.out_f != W || m.o.in_f != hv + hd) return fail(NTK_E_SHAPE, li + ": the output projections do not have the configured sizes");
+    LS_TRY(upload_vector(f, l + "o.b", W, &m.o_b));
+    if (ntk_scale(m.o_b, W, m.left_scale, stream_) != NTK_OK) return fail(NTK_E_LAUNCH, "scaling the output bias failed");
     return NTK_OK;
 }
 
@@ -414,6 +592,20 @@ int LayerStackModel::upload_mlp(const ModelFolder& f, const std::string& p, int 
 int LayerStackModel::upload_layer(const ModelFolder& f, int i, StackLayer& L) {
     const std::string p = "l" + std::to_string(i) + ".";
     const int W = info_.width;
+    if (form_.gated) {
+        LS_TRY(upload_norm(f, p + "norm1", L.norm1));
+        LS_TRY(upload_gated_mixer(f, p, i, L));
+        LS_TRY(upload_vector(f, p + "rg1.b", W, &L.rg1_b));
+        if (L.has_mlp) {
+            GatedFeedForward& G = L.gff;
+            LS_TRY(upload_norm(f, p + "norm2", L.norm2));
+            LS_TRY(upload_matrix(f, {p + "mlp.gate", p + "mlp.up", p + "rg2"}, W, G.in));
+            LS_TRY(upload_matrix(f, {p + "mlp.down"}, G.ff, G.down));
+            if (G.in.out_f != 2 * G.ff + W || G.down.out_f != W) return fail(NTK_E_SHAPE, "layer " + std::to_string(i) + ": feed-forward matrices do not have the configured sizes");
+            LS_TRY(upload_vector(f, p + "rg2.b", W, &L.rg2_b));
+        }
+        return upload_vector(f, p + "dwa", i + 2, &L.depth);
+    }
     LS_TRY(upload_norm(f, p + "norm1", L.norm1));
     if (form_.sequential) {
         LS_TRY(upload_norm(f, p + "norm1b", L.norm1b));
@@ -447,6 +639,14 @@ int LayerStackModel::load(const std::string& dir, const SeqLoadOptions& opt) {
     LS_TRY(upload_matrix(f, {"head"}, W, head_));
     if (embed_.out_f != info_.vocab || head_.out_f != info_.vocab) return fail(NTK_E_SHAPE, "embed / head do not have 'vocab' rows");
     LS_TRY(upload_norm(f, "final.norm", final_norm_));
+    if (form_.gated) {
+        const StTensor* pt = f.tensor("pos");
+        if (!pt || pt->shape.size() != 2 || pt->shape[1] != W) return fail(NTK_E_SHAPE, "tensor 'pos' is not [positions, width]");
+        LS_TRY(upload_matrix(f, {"pos"}, W, pos_));
+        n_positions_ = (int)pos_.out_f;
+        opt_.max_context = std::min(opt_.max_context, n_positions_);   // a slot holds no more positions than the table has vectors
+        LS_TRY(upload_norm(f, "embed.norm", embed_norm_));
+    }
     if (final_norm_.b && logit_scale_ != 1.0f) {   // logits = head (norm x) * scale = head (norm x with weight and bias times scale): no launch of its own per step
         if (ntk_scale(final_norm_.w, W, logit_scale_, stream_) != NTK_OK || ntk_scale(final_norm_.b, W, logit_scale_, stream_) != NTK_OK) return fail(NTK_E_LAUNCH, "scaling the output norm failed");
         logit_scale_ = 1.0f;
@@ -483,18 +683,30 @@ int LayerStackModel::alloc_buffers() {
             max_hdv_ = std::max(max_hdv_, m.heads * m.vdim);
             if (m.vdim > 512) return fail(NTK_E_SHAPE, "vdim up to 512 is supported");
             wsc = std::max(wsc, ntk_window_attention_scratch(chunk_, m.heads, m.maps, m.vdim, opt_.max_context));
-        } else {
+        } else if (L.mixer == kMixLightning) {
             const LightningMixer& m = L.lin;
             max_in_ = std::max<int>(max_in_, (int)m.in.out_f);
             max_hdv_ = std::max(max_hdv_, m.heads * m.vdim);
             lsc = std::max(lsc, ntk_lightning_attention_scratch(chunk_, m.heads, m.dim, m.vdim));
+        } else if (L.mixer == kMixGla) {
+            const GlaMixer& m = L.gla;
+            max_in_ = std::max<int>(max_in_, (int)m.in.out_f);
+            max_hdv_ = std::max(max_hdv_, m.heads * m.vdim);
+            max_rec_ = std::max(max_rec_, m.heads * m.dim);
+        } else {
+            const ParallelMixer& m = L.par;
+            max_in_ = std::max<int>(max_in_, (int)m.in.out_f);
+            max_hdv_ = std::max<int>(max_hdv_, (int)m.o.in_f);
+            max_rec_ = std::max(max_rec_, m.right.heads * m.right.dim);
+            wsc = std::max(wsc, ntk_window_attention_scratch(chunk_, m.left.heads, 1, m.left.vdim, opt_.max_context));
         }
+        if (form_.gated && L.has_mlp) max_gu2_ = std::max<int>(max_gu2_, (int)L.gff.in.out_f), max_ffn_ = std::max(max_ffn_, L.gff.ff);
         if (L.mlp_kind == kMlpMoe) {
             max_top_ = std::max(max_top_, L.mlp.top);
             max_e_ = std::max(max_e_, L.mlp.experts);
             max_ff2_ = std::max(max_ff2_, 2 * L.mlp.routed.ff);
             if (L.mlp.has_shared) max_sff2_ = std::max(max_sff2_, 2 * L.mlp.shared.ff);
-        } else if (L.mlp_kind == kMlpDense) {
+        } else if (L.mlp_kind == kMlpDense && !form_.gated) {
             max_ffn_ = std::max(max_ffn_, L.ffn.ff);
         }
     }
@@ -507,6 +719,9 @@ int LayerStackModel::alloc_buffers() {
         ok = ok && fl(&cat_, C * 2 * W) && fl(&cq_, C * std::max(max_qrank_, 1)) && fl(&q_, C * max_hqd_) && fl(&qf_, (size_t)kSharedRows * max_fold_) &&
              fl(&lat_, (size_t)kSharedRows * max_hr_) && fl(&kx_, ctx * max_hdn_) && fl(&vx_, ctx * max_hdv_) && fl(&scratch_, sc);
     if (form_.sequential) ok = ok && fl(&hist_, (C + (size_t)taps_ - 1) * W) && fl(&ff_, C * W) && fl(&zf_, C * max_ffn_) && fl(&wscratch_, wsc) && fl(&lscratch_, lsc);
+    if (form_.gated)
+        ok = ok && fl(&ff_, C * W) && fl(&zf_, C * max_ffn_) && fl(&wscratch_, wsc) && fl(&results_, (runs_.size() + 1) * C * W) && fl(&zq_, C * std::max(max_rec_, 1)) &&
+             fl(&gu2_, C * std::max(max_gu2_, 1));
     want_dev_ = tokens_dev_ ? tokens_dev_ + C : nullptr;   // one staging area: [tokens of a pass | wanted places], filled by ONE stream-ordered copy from pinned memory
     h_stage_ = (int*)nt_hip_malloc_host(2 * C * sizeof(int));
     ok = ok && h_stage_ != nullptr;
@@ -525,8 +740,8 @@ int LayerStackModel::alloc_buffers() {
             r.cache = (float*)dev_alloc((size_t)opt_.slots * ctx * row * sizeof(float));
             if (!r.cache) return fail(NTK_E_NOMEM, "out of device memory (cache)");
         }
-        if (L.mixer == kMixLightning) {
-            r.state = (float*)dev_alloc((size_t)opt_.slots * L.lin.state_floats() * sizeof(float));
+        if (L.state_floats()) {
+            r.state = (float*)dev_alloc((size_t)opt_.slots * L.state_floats() * sizeof(float));
             if (!r.state) return fail(NTK_E_NOMEM, "out of device memory (state)");
         }
         if (form_.sequential && taps_ > 1) {
@@ -654,6 +869,104 @@ int LayerStackModel::run_dense_ff(const StackLayer& L, int T) {
     return ntk_dense_linear(ff_, W, zf_, D.ff, D.down.ptr, D.down.dtype, T, W, D.ff, 0, stream_);
 }
 
+// gated linear attention: one product for [q | k | v | gate | a1 | residual gate], the decay's second projection, the recurrence (decay formed from its raw
+// projection on the way in), unit norm per head with the shared weight and the silu gate, output projection -> mix_
+int LayerStackModel::run_gla(const StackLayer& L, float* state, int T, int pos0) {
+    const GlaMixer& m = L.gla;
+    const int W = info_.width, na = (int)m.in.out_f, hq = m.heads * m.dim, hv = m.heads * m.vdim;
+    LS_TRY(ntk_dense_linear(a_, na, h1_, W, m.in.ptr, m.in.dtype, T, na, W, 0, stream_));
+    LS_TRY(ntk_dense_linear(zq_, hq, a_ + m.a_off, na, m.a2.ptr, m.a2.dtype, T, hq, m.rank, 0, stream_));
+    ntk_gated_recurrence_desc d{};
+    d.out = att_; d.ldo = hv; d.q = a_; d.ldq = na; d.k = a_ + m.k_off; d.ldk = na; d.v = a_ + m.v_off; d.ldv = na;
+    d.wz = zq_; d.ldw = hq; d.wb = m.a2_b; d.decay_form = NTK_DECAY_SIGMOID_ROOT; d.decay_param = m.tau;
+    d.state = state; d.H = m.heads; d.dn = m.dim; d.dv = m.vdim; d.q_scale = 1.0f / std::sqrt((float)m.dim); d.pos0 = pos0; d.T = T;
+    LS_TRY(ntk_gated_recurrence(&d, stream_));
+    LS_TRY(ntk_head_rmsnorm_gate(att_, hv, att_, hv, m.norm, 0, a_ + m.g_off, na, 2, 1.0f, T, m.heads, m.vdim, eps_, stream_));
+    return ntk_dense_linear(mix_, W, att_, hv, m.o.ptr, m.o.dtype, T, W, hv, 0, stream_);
+}
+
+// two mixers over the same input: one product for all their projections and the residual gate; left: biases and the query temperature on the way into the
+// cache, attention with the distance bias, sigmoid gate; right: the decay's second projection, the delta-rule recurrence, unit norm per head, weight and
+// sigmoid gate; both results side by side (each times its fixed weight) through ONE output product -> mix_
+int LayerStackModel::run_parallel(const StackLayer& L, float* cache, float* state, int T, int pos0) {
+    const ParallelMixer& m = L.par;
+    const BiasedAttention& a = m.left;
+    const DeltaMixer& r = m.right;
+    const int W = info_.width, na = (int)m.in.out_f, hv = a.heads * a.vdim, hd = r.heads * r.dim, no = hv + hd;
+    LS_TRY(ntk_dense_linear(a_, na, h1_, W, m.in.ptr, m.in.dtype, T, na, W, 0, stream_));
+    // ---- left
+    ntk_rotary rot{nullptr, 1.0f, 0};
+    LS_TRY(ntk_window_prepare_biased(cache, a.row(), a_ + a.q_off, na, a_ + a.k_off, na, a_ + a.v_off, na, a.heads, a.kv_heads, 1, a.dim, a.vdim, &rot, a.q_b, a.k_b, a.v_b,
+                                     a.temp_coef, a.temp_every, pos0, T, stream_));
+    ntk_window_attention_desc d{};
+    d.out = att_; d.ldo = no; d.q = a_ + a.q_off; d.ldq = na; d.cache = cache; d.row = a.row(); d.H = a.heads; d.G = a.kv_heads; d.maps = 1; d.dn = a.dim; d.dv = a.vdim;
+    d.pos0 = pos0; d.T = T; d.window = 0; d.scale = a.scale; d.out_scale = 1.0f; d.eps = eps_; d.scratch = wscratch_;
+    d.rel = a.rel; d.bucket_of = a.bucket_of; d.n_dist = opt_.max_context;
+    LS_TRY(ntk_window_attention(&d, stream_));
+    LS_TRY(ntk_sigmoid_gate_scaled(att_, no, a_ + a.g_off, na, nullptr, m.left_scale, T, hv, stream_));
+    // ---- right
+    LS_TRY(ntk_tanh_rows(a_ + r.w1_off, na, T, r.rank, stream_));
+    LS_TRY(ntk_dense_linear(zq_, hd, a_ + r.w1_off, na, r.w2.ptr, r.w2.dtype, T, hd, r.rank, 0, stream_));
+    ntk_gated_recurrence_desc g{};
+    g.out = att_ + hv; g.ldo = no; g.q = a_ + r.r_off; g.ldq = na; g.k = a_ + r.k_off; g.ldk = na; g.v = a_ + r.v_off; g.ldv = na;
+    g.wz = zq_; g.ldw = hd; g.wb = r.w0; g.decay_form = NTK_DECAY_EXP_SIGMOID; g.decay_param = kDeltaDecayRate;
+    g.az = a_ + r.a_off; g.lda = na; g.ab = r.a_b; g.unit_eps = kUnitKeyEps;
+    g.state = state; g.H = r.heads; g.dn = r.dim; g.dv = r.dim; g.q_scale = 1.0f; g.pos0 = pos0; g.T = T;
+    LS_TRY(ntk_gated_recurrence(&g, stream_));
+    LS_TRY(ntk_head_rmsnorm_gate(att_ + hv, no, att_ + hv, no, r.norm, r.dim, a_ + r.g_off, na, 1, m.right_scale, T, r.heads, r.dim, eps_, stream_));
+    return ntk_dense_linear(mix_, W, att_, no, m.o.ptr, m.o.dtype, T, W, no, 0, stream_);
+}
+
+// gate and up (decoding: the gated unit inside the product's launch) and the residual gate's rows, down -> ff_; the residual gate stays in gu2_ behind them
+int LayerStackModel::run_gated_ff(const StackLayer& L, int T) {
+    const GatedFeedForward& G = L.gff;
+    const int W = info_.width, n2 = (int)G.in.out_f, ff = G.ff;
+    if (T <= ntk_dense_few_rows()) {
+        ntk_dense_desc d{};
+        d.Y = zf_; d.ldy = ff; d.X = h2_; d.ldx = W; d.W = G.in.ptr; d.wdtype = G.in.dtype; d.G = 1; d.row_div = 1; d.T = T; d.N = 2 * ff; d.K = W;
+        d.glu_ff = ff; d.glu_limit = INFINITY; d.glu_alpha = kGeluAlpha; d.glu_cubic = kGeluCubic; d.glu_up_offset = 0.0f;
+        LS_TRY(ntk_dense(&d, stream_));
+        const size_t es = G.in.dtype == NTK_DT_BF16 ? 2 : 4;
+        LS_TRY(ntk_dense_linear(gu2_ + 2 * ff, n2, h2_, W, (const char*)G.in.ptr + (size_t)2 * ff * W * es, G.in.dtype, T, W, W, 0, stream_));
+    } else {
+        LS_TRY(ntk_dense_linear(gu2_, n2, h2_, W, G.in.ptr, G.in.dtype, T, n2, W, 0, stream_));
+        LS_TRY(ntk_glu_cubic(zf_, gu2_, n2, T, ff, INFINITY, kGeluAlpha, kGeluCubic, 0.0f, stream_));
+    }
+    return ntk_dense_linear(ff_, W, zf_, ff, G.down.ptr, G.down.dtype, T, W, ff, 0, stream_);
+}
+
+// A layer of the gated form.  h1_ holds the first norm of the stream already (the embedding's launch or the previous layer's last seam wrote it).  Every
+// seam is one launch: gated residual sum, after the layer's last sublayer the weighted sum over all layer results so far, and the norm that follows.
+int LayerStackModel::gated_layer(size_t r, const StackLayer& L, int slot, int T, int pos0) {
+    const int W = info_.width;
+    const Run& run = runs_[r];
+    const NormW* next = r + 1 < runs_.size() ? &layers_[(size_t)runs_[r + 1].layer].norm1 : nullptr;
+    float* state = run.state + (size_t)slot * L.state_floats();
+    int na, rg_off;
+    const float* yb = nullptr;
+    if (L.mixer == kMixGla) {
+        LS_TRY(run_gla(L, state, T, pos0));
+        na = (int)L.gla.in.out_f; rg_off = L.gla.rg_off;
+    } else {
+        LS_TRY(run_parallel(L, run.cache + (size_t)slot * opt_.max_context * L.par.left.row(), state, T, pos0));
+        na = (int)L.par.in.out_f; rg_off = L.par.rg_off; yb = L.par.o_b;
+    }
+    auto depth = [&](ntk_gated_seam_desc& d) {     // the layer's result joins the others; what goes on is their weighted sum, normed for the next layer
+        d.hist = results_; d.hist_stride = (long long)chunk_ * W; d.n_hist = run.layer + 2; d.coef = L.depth;
+        if (next) { d.h = h1_; d.ldh = W; d.nw = next->w; d.nb = next->b; d.alpha = next->alpha; }
+    };
+    ntk_gated_seam_desc d{};
+    d.x = x_; d.ldx = W; d.y = mix_; d.ldy = W; d.yb = yb; d.g = a_ + rg_off; d.ldg = na; d.gb = L.rg1_b; d.T = T; d.n = W;
+    if (!L.has_mlp) { depth(d); return ntk_gated_seam(&d, stream_); }
+    d.h = h2_; d.ldh = W; d.nw = L.norm2.w; d.nb = L.norm2.b; d.alpha = L.norm2.alpha;
+    LS_TRY(ntk_gated_seam(&d, stream_));
+    LS_TRY(run_gated_ff(L, T));
+    ntk_gated_seam_desc e{};
+    e.x = x_; e.ldx = W; e.y = ff_; e.ldy = W; e.g = gu2_ + 2 * L.gff.ff; e.ldg = (int)L.gff.in.out_f; e.gb = L.rg2_b; e.T = T; e.n = W;
+    depth(e);
+    return ntk_gated_seam(&e, stream_);
+}
+
 // out = h + conv(h), h = layer norm of the stream: the carried inputs in front of the portion's, the convolution, and the portion's last inputs carried on
 // The sublayer output that the stream has not taken yet (owed_) goes in first, in the same launch: the norm after one sublayer and the norm before the next
 // read the same row.  One token: one launch for the whole seam.
@@ -705,6 +1018,13 @@ int LayerStackModel::portion(int slot, const int* tokens_dev, int T, int pos0, c
     const int W = info_.width;
     // (the embedding is kept beside the stream only where a repeated span is entered through a projection of both)
     const bool keep_embedding = has_loop_ && form_.loop_projection;
+    if (form_.gated) {
+        // token row + position row, the embedding's norm; the result is the first of the layer results; then the first layer's norm
+        LS_TRY(ntk_embed_positions(x_, results_, embed_.ptr, pos_.ptr, embed_.dtype, tokens_dev, T, info_.vocab, W, pos0, n_positions_, embed_norm_.w, embed_norm_.b,
+                                   embed_norm_.alpha, stream_));
+        const NormW& n1 = layers_[(size_t)runs_[0].layer].norm1;
+        LS_TRY(ntk_dyt(h1_, W, x_, W, n1.w, n1.b, n1.alpha, T, W, stream_));
+    } else
     LS_TRY(ntk_embed_dense_scaled(keep_embedding ? x0_ : x_, embed_.ptr, embed_.dtype, tokens_dev, T, info_.vocab, W, embed_scale_, stream_));
     bool x_is_x0 = keep_embedding;   // until the first layer run writes x_
     owed_.y = nullptr;
@@ -717,7 +1037,9 @@ int LayerStackModel::portion(int slot, const int* tokens_dev, int T, int pos0, c
             LS_TRY(ntk_dense_linear(x_, W, cat_, 2 * W, loop_in_.ptr, loop_in_.dtype, T, W, 2 * W, 0, stream_));
             x_is_x0 = false;
         }
-        if (form_.sequential) {
+        if (form_.gated) {
+            LS_TRY(gated_layer(r, L, slot, T, pos0));
+        } else if (form_.sequential) {
             LS_TRY(sequential_layer(run, L, slot, T, pos0));
             if (r + 1 == runs_.size() || (capture_ && capture_buf_)) LS_TRY(settle(T));
         } else {
@@ -733,7 +1055,8 @@ int LayerStackModel::portion(int slot, const int* tokens_dev, int T, int pos0, c
         ntk_dense_desc d{};
         d.Y = logits_out; d.ldy = info_.vocab; d.X = rows; d.ldx = W; d.W = head_.ptr; d.wdtype = head_.dtype; d.G = 1; d.row_div = 1; d.T = n_want;
         d.N = info_.vocab; d.K = W;
-        if (final_norm_.b) { LS_TRY(ntk_layernorm(hn_, W, rows, W, final_norm_.w, final_norm_.b, n_want, W, eps_, 0, stream_)); d.X = hn_; }
+        if (form_.gated) { LS_TRY(ntk_dyt(hn_, W, rows, W, final_norm_.w, final_norm_.b, final_norm_.alpha, n_want, W, stream_)); d.X = hn_; }
+        else if (final_norm_.b) { LS_TRY(ntk_layernorm(hn_, W, rows, W, final_norm_.w, final_norm_.b, n_want, W, eps_, 0, stream_)); d.X = hn_; }
         else if (n_want <= ntk_dense_few_rows()) { d.norm_w = final_norm_.w; d.norm_eps = eps_; d.norm_offset = 1.0f; }   // the output norm inside the head's launch
         else { LS_TRY(ntk_rmsnorm_offset(hn_, final_norm_.w, nullptr, nullptr, W, rows, W, n_want, W, eps_, 1.0f, stream_)); d.X = hn_; }
         LS_TRY(ntk_dense(&d, stream_));

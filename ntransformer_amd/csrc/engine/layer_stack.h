@@ -6,6 +6,10 @@
 //   sequential   x += norm1b(mixer(conv(norm1 x))), then x += norm2b(ff(conv(norm2 x))): layer norms with weight and bias before and after every
 //                sublayer, a short causal convolution added to every sublayer's input (its last inputs are part of a sequence's state), scaled
 //                embedding and logits                                                                                       -- "Nizorax"
+//   gated        pre-norm, x += gate * mixer(norm1 x), then x += gate * ff(norm2 x): dynamic-tanh norms (element by element, no row sums), every sublayer's
+//                result multiplied by sigmoid(W h + b) of the sublayer's input before it joins the stream, the stream that goes on after a layer a
+//                learned weighted sum of ALL layer results so far (and the embedding), a learned vector per position added to the embedding, scaled
+//                logits                                                                                                     -- "Tubazen"
 //
 // Mechanisms are parsed into parameter structs and run by the operators of include/ntk_layers.h, so another family can list them in another order
 // or with other constants:
@@ -13,8 +17,13 @@
 //                 one matrix, sliding window): one LatentMixer each -- which of the options a layer has is read from its config keys;
 //                 "attention": grouped-query attention over rotated keys with a sliding window, as a differential pair of score maps when the
 //                 config gives 'diff' (WindowMixer); "lightning": linear attention with a per-head decay and a recurrent state (LightningMixer);
+//                 "gla": gated linear attention -- a recurrent state that forgets per token and key channel (decay from a low-rank projection), unit norm
+//                 per head, silu gate (GlaMixer); "parallel": two mixers over the same input whose results are added with fixed weights -- grouped-query
+//                 softmax attention with projection biases, a query temperature growing with the position and a learned bias by bucketed distance
+//                 (BiasedAttention), beside a delta-rule recurrence with per-channel decay and removal rate (DeltaMixer);
 //   feed-forward  kind "moe": routed gated experts + an optional shared expert (MoeFeedForward: softmax or sigmoid scores, optional expert groups,
-//                 clipped or plain gated units); kind "dense": up, polynomial activation with unit-norm terms, down (DenseFeedForward).
+//                 clipped or plain gated units); kind "dense": up, polynomial activation with unit-norm terms, down (DenseFeedForward), or in the
+//                 gated form a gated unit with the tanh form of gelu (GatedFeedForward).
 // What a sequence holds per layer run: cache rows per position (attention kinds), a recurrent state (lightning), the convolutions' last inputs.
 #pragma once
 #include <string>
@@ -72,6 +81,53 @@ struct LightningMixer {               // linear attention with a per-head decay;
     size_t state_floats() const { return (size_t)heads * dim * vdim; }
 };
 
+struct GlaMixer {                     // gated linear attention: S = diag(alpha_t) S + k v^T, alpha = sigmoid(W_a2 W_a1 h + b)^(1 / tau) per key channel
+    int heads = 0, dim = 0, vdim = 0, rank = 0;
+    float tau = 1.0f;
+    DenseW in;                        // rows [q | k | v | gate | a1 | residual gate]
+    int k_off = 0, v_off = 0, g_off = 0, a_off = 0, rg_off = 0;
+    DenseW a2;                        // [heads * dim][rank]
+    float* a2_b = nullptr;            // F32 [heads * dim]
+    float* norm = nullptr;            // F32 [vdim], shared by the heads
+    DenseW o;
+    size_t state_floats() const { return (size_t)heads * dim * vdim; }
+};
+
+struct BiasedAttention {              // grouped-query softmax attention, causal, no rotation: biases on q / k / v / o, query temperature, bias by bucketed distance
+    int heads = 0, kv_heads = 0, dim = 0, vdim = 0, buckets = 0;
+    float scale = 1.0f, temp_coef = 0.0f;
+    double temp_every = 1.0, bias_max = 1.0;
+    float *q_b = nullptr, *k_b = nullptr, *v_b = nullptr;
+    float* rel = nullptr;             // F32 [buckets][heads]
+    int* bucket_of = nullptr;         // device int [slot capacity]: bucket of every distance
+    int q_off = 0, k_off = 0, v_off = 0, g_off = 0;
+    int row() const { return kv_heads * (dim + vdim); }
+};
+
+struct DeltaMixer {                   // S = diag(w) S - (a u)(u^T S) + k v^T, w = exp(-e^(-1/2) sigmoid(W_w2 tanh(W_w1 h) + w0)), a = sigmoid(W_a h + b), u the unit key
+    int heads = 0, dim = 0, rank = 0;
+    int r_off = 0, k_off = 0, v_off = 0, g_off = 0, a_off = 0, w1_off = 0;
+    DenseW w2;                        // [heads * dim][rank]
+    float *w0 = nullptr, *a_b = nullptr, *norm = nullptr;   // F32 [heads * dim] each
+    size_t state_floats() const { return (size_t)heads * dim * dim; }
+};
+
+struct ParallelMixer {                // left_scale * attention + right_scale * delta rule, both over the same input
+    BiasedAttention left;
+    DeltaMixer right;
+    float left_scale = 1.0f, right_scale = 1.0f;
+    DenseW in;                        // rows [left q | k | v | gate | right r | k | v | gate | a | w1 | residual gate] of one product
+    int rg_off = 0;
+    DenseW o;                         // [width][left heads * vdim + right heads * dim]: both output projections side by side
+    float* o_b = nullptr;             // F32 [width]: left_scale * the left output bias
+};
+
+struct GatedFeedForward {             // down(gelu_tanh(gate h) * (up h)), its result gated like the mixer's
+    int ff = 0;
+    DenseW in;                        // rows [gate | up | residual gate]
+    DenseW down;
+};
+
 struct GatedExperts {                 // `count` experts of the same shape, stacked: gate rows then up rows, and the down matrices
     int ff = 0;
     float limit = 0.0f;               // clamp of the gate (from above) and the up value (both sides); INFINITY: none
@@ -95,9 +151,9 @@ struct DenseFeedForward {             // down(act(up h)), act = a N(z) + b N(z^2
     float* act = nullptr;             // F32 [4]
 };
 
-struct NormW { float* w = nullptr; float* b = nullptr; };   // b: layer norm with bias (sequential form); none: RMS norm, weight around zero
+struct NormW { float* w = nullptr; float* b = nullptr; float alpha = 0.0f; };   // b: layer norm with bias (sequential form) / dynamic tanh with its alpha (gated form); none: RMS norm, weight around zero
 
-enum MixerKind { kMixLatent = 0, kMixWindow = 1, kMixLightning = 2 };
+enum MixerKind { kMixLatent = 0, kMixWindow = 1, kMixLightning = 2, kMixGla = 3, kMixParallel = 4 };
 enum MlpKind { kMlpNone = 0, kMlpMoe = 1, kMlpDense = 2 };
 
 struct StackLayer {
@@ -109,16 +165,23 @@ struct StackLayer {
     LatentMixer mix;
     WindowMixer att;
     LightningMixer lin;
+    GlaMixer gla;
+    ParallelMixer par;
+    GatedFeedForward gff;
+    float *rg1_b = nullptr, *rg2_b = nullptr;   // gated form: biases of the residual gates, F32 [width]
+    float* depth = nullptr;                 // gated form: weights of the layer results so far (embedding first), device F32 [layer + 2]
     int mlp_kind = kMlpNone;
     bool has_mlp = false;
     MoeFeedForward mlp;
     DenseFeedForward ffn;
-    int cache_row() const { return mixer == kMixLatent ? mix.row() : mixer == kMixWindow ? att.row() : 0; }
+    int cache_row() const { return mixer == kMixLatent ? mix.row() : mixer == kMixWindow ? att.row() : mixer == kMixParallel ? par.left.row() : 0; }
+    size_t state_floats() const { return mixer == kMixLightning ? lin.state_floats() : mixer == kMixGla ? gla.state_floats() : mixer == kMixParallel ? par.right.state_floats() : 0; }
 };
 
 // what a family fixes about its layers (everything else is read from config.json)
 struct StackForm {
     bool sequential = false;          // see the head of this file
+    bool gated = false;               // ... (neither: the parallel form)
     bool loop_projection = true;      // the repeated span is entered through 'loop.in' over [stream ; embedding]
     int router_score = 0;             // 0 softmax, 1 sigmoid
     bool router_renorm = true;
@@ -154,6 +217,15 @@ private:
     int parse_mixer(const Json& L, const std::string& type, LatentMixer& m);
     int parse_window(const Json& L, WindowMixer& m);
     int parse_lightning(const Json& L, LightningMixer& m);
+    int parse_gla(const Json& L, GlaMixer& m);
+    int parse_parallel(const Json& L, ParallelMixer& m);
+    int upload_gated_mixer(const ModelFolder& f, const std::string& p, int i, StackLayer& L);
+    int upload_hstack(const ModelFolder& f, const std::vector<std::string>& names, DenseW& out);
+    int read_scalar(const ModelFolder& f, const std::string& name, float* out);
+    int run_gla(const StackLayer& L, float* state, int T, int pos0);
+    int run_parallel(const StackLayer& L, float* cache, float* state, int T, int pos0);
+    int run_gated_ff(const StackLayer& L, int T);
+    int gated_layer(size_t r, const StackLayer& L, int slot, int T, int pos0);
     int parse_mlp(const Json& ml, const std::string& where, StackLayer& S);
     int upload_norm(const ModelFolder& f, const std::string& name, NormW& out);
     int upload_mixer(const ModelFolder& f, const std::string& p, int i, StackLayer& L);
@@ -189,7 +261,9 @@ private:
     std::vector<StackLayer> layers_;
     std::vector<Run> runs_;
     bool has_loop_ = false;
-    DenseW embed_, head_, loop_in_;
+    DenseW embed_, head_, loop_in_, pos_;   // pos_: a learned vector per position (gated form)
+    NormW embed_norm_;
+    int n_positions_ = 0;             // rows of the position table
     NormW final_norm_;
     uint64_t weight_bytes_ = 0;
     std::vector<void*> allocs_;
@@ -201,7 +275,9 @@ private:
     // activations
     float *x_ = nullptr, *x0_ = nullptr, *cat_ = nullptr, *h1_ = nullptr, *h2_ = nullptr, *a_ = nullptr, *cq_ = nullptr, *q_ = nullptr, *qf_ = nullptr, *lat_ = nullptr,
           *att_ = nullptr, *kx_ = nullptr, *vx_ = nullptr, *mix_ = nullptr, *wts_ = nullptr, *sg_ = nullptr, *gu_ = nullptr, *act_ = nullptr, *dn_ = nullptr,
-          *sgu_ = nullptr, *sact_ = nullptr, *sdn_ = nullptr, *scratch_ = nullptr, *xw_ = nullptr, *hn_ = nullptr, *hist_ = nullptr, *ff_ = nullptr, *zf_ = nullptr, *wscratch_ = nullptr, *lscratch_ = nullptr;
+          *sgu_ = nullptr, *sact_ = nullptr, *sdn_ = nullptr, *scratch_ = nullptr, *xw_ = nullptr, *hn_ = nullptr, *hist_ = nullptr, *ff_ = nullptr, *zf_ = nullptr, *wscratch_ = nullptr, *lscratch_ = nullptr,
+          *results_ = nullptr, *zq_ = nullptr, *gu2_ = nullptr;   // gated form: the layer results of the pass [runs + 1][chunk][width], decay pre-activations, [gate | up | residual gate]
+    int max_rec_ = 0, max_gu2_ = 0;
     int *ids_ = nullptr, *offsets_ = nullptr, *order_ = nullptr, *where_ = nullptr, *tokens_dev_ = nullptr, *want_dev_ = nullptr;
     int* h_stage_ = nullptr;          // pinned: tokens and wanted places of the pass being launched
     float* logits_ = nullptr;

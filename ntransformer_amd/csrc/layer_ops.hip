@@ -323,3 +323,168 @@ int ntk_gated_rmsnorm(float* y, int ldy, const float* x, int ldx, const float* w
     hipLaunchKernelGGL(gated_rmsnorm_kernel, dim3(T), dim3(T <= kFewRows ? 1024 : 256), 0, resolve_stream(stream), y, ldy, x, ldx, w, g, ldg, n, eps);
     return last_launch_status();
 }
+
+// ---------------------------------------------------------------------------------------------------------------- layers with gated residuals
+// The dynamic-tanh norm is element by element (no row sums), so it rides in whatever launch produces its input: the embedding (token row + position row),
+// and the seam between sublayers (gated residual sum, the average over the layer results so far, the next norm).
+namespace ntk {
+
+__device__ __forceinline__ float sigmoidf_(float z) { return 1.0f / (1.0f + expf(-z)); }
+
+__global__ void dyt_kernel(float* y, int ldy, const float* x, int ldx, const float* w, const float* b, float alpha, int n) {
+    const long long t = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    y[t * ldy + i] = fmaf(tanhf(alpha * x[t * ldx + i]), w[i], b ? b[i] : 0.0f);
+}
+
+template <typename TT>
+__global__ void embed_positions_kernel(float* out, float* copy, const TT* table, const TT* pos_table, const int* tokens, int vocab, int width, int pos0, int n_pos,
+                                       const float* w, const float* b, float alpha) {
+    const long long t = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= width) return;
+    const int tok = tokens[t];
+    const long long p = pos0 + t;
+    float e = 0.0f, pv = 0.0f;
+    if (tok >= 0 && tok < vocab) {
+        if constexpr (sizeof(TT) == 2) e = __uint_as_float((uint32_t)table[(long long)tok * width + i] << 16); else e = table[(long long)tok * width + i];
+    }
+    if (p < n_pos) {
+        if constexpr (sizeof(TT) == 2) pv = __uint_as_float((uint32_t)pos_table[p * width + i] << 16); else pv = pos_table[p * width + i];
+    }
+    float v = e + pv;
+    if (w) v = fmaf(tanhf(alpha * v), w[i], b ? b[i] : 0.0f);
+    out[t * width + i] = v;
+    if (copy) copy[t * width + i] = v;
+}
+
+__global__ void sigmoid_gate_scaled_kernel(float* y, int ldy, const float* g, int ldg, const float* gb, float scale, int n) {
+    const long long t = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    y[t * ldy + i] = y[t * ldy + i] * sigmoidf_(g[t * ldg + i] + (gb ? gb[i] : 0.0f)) * scale;
+}
+
+__global__ void tanh_rows_kernel(float* x, int ldx, int n) {
+    const long long t = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[t * ldx + i] = tanhf(x[t * ldx + i]);
+}
+
+// one wave per (token, head): the head's dv values in registers (dv <= 64 * 16), mean of squares over the wave, weight, gate
+constexpr int HRN_MAXC = 16;
+__global__ __launch_bounds__(64) void head_rmsnorm_gate_kernel(float* y, int ldy, const float* x, int ldx, const float* w, int w_head_stride, const float* g, int ldg,
+                                                               int act, float scale, int H, int dv, float eps) {
+    const int lane = threadIdx.x, h = blockIdx.x % H;
+    const long long t = blockIdx.x / H;
+    const float* xr = x + t * ldx + (long long)h * dv;
+    float v[HRN_MAXC];
+    float ss = 0.0f;
+#pragma unroll
+    for (int c = 0; c < HRN_MAXC; ++c) {
+        v[c] = c * 64 + lane < dv ? xr[c * 64 + lane] : 0.0f;
+        ss = fmaf(v[c], v[c], ss);
+    }
+    const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)dv + eps);
+#pragma unroll
+    for (int c = 0; c < HRN_MAXC; ++c) {
+        const int i = c * 64 + lane;
+        if (i >= dv) continue;
+        float r = v[c] * inv * w[(long long)h * w_head_stride + i];
+        if (act) {
+            const float gg = g[t * ldg + (long long)h * dv + i];
+            r *= act == 1 ? sigmoidf_(gg) : gg * sigmoidf_(gg);
+        }
+        y[t * ldy + (long long)h * dv + i] = r * scale;
+    }
+}
+
+struct SeamArgs {
+    float* x; int ldx;
+    const float* y; int ldy; const float* yb;
+    const float* g; int ldg; const float* gb;
+    float* hist; long long hist_stride; int n_hist; const float* coef;
+    float* h; int ldh; const float* nw; const float* nb; float alpha;
+    int n;
+};
+__global__ void gated_seam_kernel(const SeamArgs a) {
+    const long long t = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= a.n) return;
+    float r = a.x[t * a.ldx + i];
+    if (a.y) {
+        const float yy = a.y[t * a.ldy + i] + (a.yb ? a.yb[i] : 0.0f);
+        r = fmaf(yy, sigmoidf_(a.g[t * a.ldg + i] + (a.gb ? a.gb[i] : 0.0f)), r);
+    }
+    if (a.n_hist > 0) {
+        float s = 0.0f;
+        for (int j = 0; j + 1 < a.n_hist; ++j) s = fmaf(a.coef[j], a.hist[j * a.hist_stride + t * a.n + i], s);
+        a.hist[(a.n_hist - 1) * a.hist_stride + t * a.n + i] = r;
+        r = fmaf(a.coef[a.n_hist - 1], r, s);
+    }
+    a.x[t * a.ldx + i] = r;
+    if (a.h) a.h[t * a.ldh + i] = fmaf(tanhf(a.alpha * r), a.nw[i], a.nb ? a.nb[i] : 0.0f);
+}
+
+}  // namespace ntk
+
+int ntk_dyt(float* y, int ldy, const float* x, int ldx, const float* w, const float* b, float alpha, int T, int n, void* stream) {
+    if (!y || !x || !w) return NTK_E_NULL;
+    if (T < 0 || n <= 0 || ldy < n || ldx < n) return NTK_E_SHAPE;
+    if (T == 0) return NTK_OK;
+    hipLaunchKernelGGL(ntk::dyt_kernel, dim3((n + 255) / 256, T), dim3(256), 0, resolve_stream(stream), y, ldy, x, ldx, w, b, alpha, n);
+    return last_launch_status();
+}
+
+int ntk_embed_positions(float* out, float* copy, const void* table, const void* pos_table, int tdtype, const int* tokens, int T, int vocab, int width, int pos0,
+                        int n_pos, const float* w, const float* b, float alpha, void* stream) {
+    if (!out || !table || !pos_table || !tokens) return NTK_E_NULL;
+    if (tdtype != NTK_DT_BF16 && tdtype != NTK_DT_F32) return NTK_E_DTYPE;
+    if (T < 0 || vocab <= 0 || width <= 0 || pos0 < 0 || n_pos < 0) return NTK_E_SHAPE;
+    if (T == 0) return NTK_OK;
+    const dim3 grid((width + 255) / 256, T);
+    if (tdtype == NTK_DT_BF16)
+        hipLaunchKernelGGL(ntk::embed_positions_kernel<uint16_t>, grid, dim3(256), 0, resolve_stream(stream), out, copy, (const uint16_t*)table, (const uint16_t*)pos_table,
+                           tokens, vocab, width, pos0, n_pos, w, b, alpha);
+    else
+        hipLaunchKernelGGL(ntk::embed_positions_kernel<float>, grid, dim3(256), 0, resolve_stream(stream), out, copy, (const float*)table, (const float*)pos_table, tokens,
+                           vocab, width, pos0, n_pos, w, b, alpha);
+    return last_launch_status();
+}
+
+int ntk_sigmoid_gate_scaled(float* y, int ldy, const float* g, int ldg, const float* gb, float scale, int T, int n, void* stream) {
+    if (!y || !g) return NTK_E_NULL;
+    if (T < 0 || n <= 0 || ldy < n || ldg < n) return NTK_E_SHAPE;
+    if (T == 0) return NTK_OK;
+    hipLaunchKernelGGL(ntk::sigmoid_gate_scaled_kernel, dim3((n + 255) / 256, T), dim3(256), 0, resolve_stream(stream), y, ldy, g, ldg, gb, scale, n);
+    return last_launch_status();
+}
+
+int ntk_tanh_rows(float* x, int ldx, int T, int n, void* stream) {
+    if (!x) return NTK_E_NULL;
+    if (T < 0 || n <= 0 || ldx < n) return NTK_E_SHAPE;
+    if (T == 0) return NTK_OK;
+    hipLaunchKernelGGL(ntk::tanh_rows_kernel, dim3((n + 255) / 256, T), dim3(256), 0, resolve_stream(stream), x, ldx, n);
+    return last_launch_status();
+}
+
+int ntk_head_rmsnorm_gate(float* y, int ldy, const float* x, int ldx, const float* w, int w_head_stride, const float* g, int ldg, int act, float scale, int T, int H,
+                          int dv, float eps, void* stream) {
+    if (!y || !x || !w || (act && !g)) return NTK_E_NULL;
+    if (T < 0 || H <= 0 || dv <= 0 || dv > 64 * ntk::HRN_MAXC || act < 0 || act > 2 || ldy < H * dv || ldx < H * dv || (act && ldg < H * dv)) return NTK_E_SHAPE;
+    if (w_head_stride != 0 && w_head_stride != dv) return NTK_E_SHAPE;
+    if (T == 0) return NTK_OK;
+    hipLaunchKernelGGL(ntk::head_rmsnorm_gate_kernel, dim3(T * H), dim3(64), 0, resolve_stream(stream), y, ldy, x, ldx, w, w_head_stride, g, ldg, act, scale, H, dv, eps);
+    return last_launch_status();
+}
+
+int ntk_gated_seam(const ntk_gated_seam_desc* d, void* stream) {
+    if (!d || !d->x || (d->y && !d->g) || (d->n_hist > 0 && (!d->hist || !d->coef)) || (d->h && !d->nw)) return NTK_E_NULL;
+    if (d->T < 0 || d->n <= 0 || d->ldx < d->n || (d->y && (d->ldy < d->n || d->ldg < d->n)) || (d->h && d->ldh < d->n) || d->n_hist < 0) return NTK_E_SHAPE;
+    if (d->n_hist > 0 && d->hist_stride < (long long)d->T * d->n) return NTK_E_SHAPE;
+    if (d->T == 0) return NTK_OK;
+    ntk::SeamArgs a{d->x, d->ldx, d->y, d->ldy, d->yb, d->g, d->ldg, d->gb, d->hist, d->hist_stride, d->n_hist, d->coef, d->h, d->ldh, d->nw, d->nb, d->alpha, d->n};
+    hipLaunchKernelGGL(ntk::gated_seam_kernel, dim3((d->n + 255) / 256, d->T), dim3(256), 0, resolve_stream(stream), a);
+    return last_launch_status();
+}

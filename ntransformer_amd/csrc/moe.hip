@@ -189,13 +189,14 @@ __global__ __launch_bounds__(kGroupThreads) void moe_group_kernel(int* offsets, 
     }
 }
 
-__global__ void clipped_glu_kernel(float* a, const float* gu, int ff, float limit, float alpha, float up_offset) {
+__global__ void clipped_glu_kernel(float* a, const float* gu, int ldgu, int ff, float limit, float alpha, float cubic, float up_offset) {
     const long long r = blockIdx.y;
     const int f = blockIdx.x * blockDim.x + threadIdx.x;
     if (f >= ff) return;
-    const float g = fminf(gu[r * 2 * ff + f], limit);
-    const float u = fminf(fmaxf(gu[r * 2 * ff + ff + f], -limit), limit);
-    a[r * ff + f] = g * (1.0f / (1.0f + expf(-alpha * g))) * (u + up_offset);
+    const float g = fminf(gu[r * ldgu + f], limit);
+    const float u = fminf(fmaxf(gu[r * ldgu + ff + f], -limit), limit);
+    const float z = cubic != 0.0f ? fmaf(cubic * g * g, g, g) : g;
+    a[r * ff + f] = g * (1.0f / (1.0f + expf(-alpha * z))) * (u + up_offset);
 }
 
 template <bool ADD>
@@ -252,7 +253,15 @@ int ntk_glu(float* a, const float* gu, int rows, int ff, float limit, float alph
     if (!a || !gu) return NTK_E_NULL;
     if (rows < 0 || ff <= 0) return NTK_E_SHAPE;
     if (rows == 0) return NTK_OK;
-    hipLaunchKernelGGL(clipped_glu_kernel, dim3((ff + 255) / 256, rows), dim3(256), 0, resolve_stream(stream), a, gu, ff, limit, alpha, up_offset);
+    hipLaunchKernelGGL(clipped_glu_kernel, dim3((ff + 255) / 256, rows), dim3(256), 0, resolve_stream(stream), a, gu, 2 * ff, ff, limit, alpha, 0.0f, up_offset);
+    return last_launch_status();
+}
+
+int ntk_glu_cubic(float* a, const float* gu, int ldgu, int rows, int ff, float limit, float alpha, float cubic, float up_offset, void* stream) {
+    if (!a || !gu) return NTK_E_NULL;
+    if (rows < 0 || ff <= 0 || ldgu < 2 * ff) return NTK_E_SHAPE;
+    if (rows == 0) return NTK_OK;
+    hipLaunchKernelGGL(clipped_glu_kernel, dim3((ff + 255) / 256, rows), dim3(256), 0, resolve_stream(stream), a, gu, ldgu, ff, limit, alpha, cubic, up_offset);
     return last_launch_status();
 }
 

@@ -13,11 +13,19 @@
 namespace ntk {
 
 // one workgroup per token: q rotated in place, k rotated into the cache row, v copied behind.  Angles in double (position times frequency), applied in F32.
+// Optional: what the projections left to their consumer -- bias vectors on q, k and v, and a query temperature that grows with the position.
 __global__ __launch_bounds__(256) void window_prepare_kernel(float* cache, int row, float* q, int ldq, const float* k, int ldk, const float* v, int ldv, int nq, int nk,
-                                                             int dn, int nv, const double* freq, float mag, int dims, int pos0) {
+                                                             int dn, int nv, const double* freq, float mag, int dims, int pos0, const float* qb, const float* kb,
+                                                             const float* vb, float temp_coef, double temp_every) {
     extern __shared__ float cs[];   // [dims / 2] cos, [dims / 2] sin
     const int t = blockIdx.x, pos = pos0 + t;
     const int half = dims / 2;
+    if (qb || temp_coef != 0.0f) {     // (uniform over the launch) q = (q + bias) * temperature, ahead of the rotation: a thread rewrites its own entries
+        float* qt0 = q + (long long)t * ldq;
+        const float temp = temp_coef != 0.0f ? 1.0f + temp_coef * logf((float)floor((double)(pos + 1) / temp_every) + 1.0f) : 1.0f;
+        for (int j = threadIdx.x; j < nq * dn; j += 256) qt0[j] = (qt0[j] + (qb ? qb[j] : 0.0f)) * temp;
+        __syncthreads();
+    }
     for (int i = threadIdx.x; i < half; i += 256) {
         const double a = (double)pos * freq[i];
         cs[i] = (float)(cos(a) * (double)mag);
@@ -38,16 +46,16 @@ __global__ __launch_bounds__(256) void window_prepare_kernel(float* cache, int r
     for (int j = threadIdx.x; j < nk * half; j += 256) {
         const int o = (j / half) * dn + 2 * (j % half);
         float ra, rb;
-        rope_rotate(kt[o], kt[o + 1], cs[j % half], cs[half + j % half], ra, rb);
+        rope_rotate(kt[o] + (kb ? kb[o] : 0.0f), kt[o + 1] + (kb ? kb[o + 1] : 0.0f), cs[j % half], cs[half + j % half], ra, rb);
         dst[o] = ra;
         dst[o + 1] = rb;
     }
     const int rest = dn - dims;
     for (int j = threadIdx.x; j < nk * rest; j += 256) {
         const int o = (j / rest) * dn + dims + j % rest;
-        dst[o] = kt[o];
+        dst[o] = kt[o] + (kb ? kb[o] : 0.0f);
     }
-    for (int j = threadIdx.x; j < nv; j += 256) dst[nk * dn + j] = vt[j];
+    for (int j = threadIdx.x; j < nv; j += 256) dst[nk * dn + j] = vt[j] + (vb ? vb[j] : 0.0f);
 }
 
 struct WinArgs {
@@ -58,6 +66,7 @@ struct WinArgs {
     float scale, lambda;
     int sub_norm; float eps, out_scale;
     int splits; float* scratch;       // splits > 1: states [T * H][splits][maps][2 + dv]
+    const float* rel; const int* bucket_of; int n_dist;   // rel != NULL: rel[bucket_of[min(distance, n_dist - 1)] * H + head] joins the scaled score
 };
 
 constexpr int WROWS = 16, WQPW = 4, WKCH = 64, WSLAB = 64, WMAXC = 8;   // dv <= WMAXC * WSLAB
@@ -110,11 +119,12 @@ __global__ __launch_bounds__(256) void window_attention_kernel(const WinArgs a) 
             if (e0 + 256 * u < WROWS * M * DNP) Qs[e0 + 256 * u] = qv[u];
     }
     float mx[M][WQPW], l[M][WQPW], acc[M][WQPW][WMAXC];
-    int rpos[WQPW];
+    int rpos[WQPW], rhead[WQPW];
 #pragma unroll
     for (int i = 0; i < WQPW; ++i) {
         const int rho = row0 + wave * WQPW + i;
         rpos[i] = rho < n_rows ? a.pos0 + rho / R : -1;
+        rhead[i] = g * R + rho % R;
 #pragma unroll
         for (int m = 0; m < M; ++m) {
             mx[m][i] = -INFINITY; l[m][i] = 0.0f;
@@ -163,7 +173,8 @@ __global__ __launch_bounds__(256) void window_attention_kernel(const WinArgs a) 
 #pragma unroll
             for (int i = 0; i < WQPW; ++i) {
                 const bool vis = lane < nk && rpos[i] >= 0 && j <= rpos[i] && (a.window <= 0 || rpos[i] - j < a.window);
-                const float sv = vis ? s[i] * a.scale : -INFINITY;
+                float sv = vis ? s[i] * a.scale : -INFINITY;
+                if (a.rel && vis) sv += a.rel[(long long)a.bucket_of[min(rpos[i] - j, a.n_dist - 1)] * a.H + rhead[i]];
                 const float mn = fmaxf(mx[m][i], wave_max(sv));
                 const float ms = mn == -INFINITY ? 0.0f : mn;
                 const float p = vis ? expf(sv - ms) : 0.0f;
@@ -296,13 +307,20 @@ using namespace ntk;
 
 int ntk_window_prepare(float* cache, int row, float* q, int ldq, const float* k, int ldk, const float* v, int ldv, int H, int G, int maps, int dn, int dv,
                        const ntk_rotary* rot, int pos0, int T, void* stream) {
+    return ntk_window_prepare_biased(cache, row, q, ldq, k, ldk, v, ldv, H, G, maps, dn, dv, rot, nullptr, nullptr, nullptr, 0.0f, 1.0, pos0, T, stream);
+}
+
+int ntk_window_prepare_biased(float* cache, int row, float* q, int ldq, const float* k, int ldk, const float* v, int ldv, int H, int G, int maps, int dn, int dv,
+                              const ntk_rotary* rot, const float* qb, const float* kb, const float* vb, float temp_coef, double temp_every, int pos0, int T,
+                              void* stream) {
     if (!cache || !q || !k || !v || !rot || (rot->dims > 0 && !rot->freq)) return NTK_E_NULL;
+    if (temp_coef != 0.0f && !(temp_every > 0.0)) return NTK_E_SHAPE;
     if (T < 0 || H <= 0 || G <= 0 || H % G || maps < 1 || dn <= 0 || dv <= 0 || pos0 < 0) return NTK_E_SHAPE;
     if (rot->dims < 0 || (rot->dims & 1) || rot->dims > dn) return NTK_E_SHAPE;
     if (row < G * (maps * dn + dv) || ldq < H * maps * dn || ldk < G * maps * dn || ldv < G * dv) return NTK_E_SHAPE;
     if (T == 0) return NTK_OK;
     hipLaunchKernelGGL(window_prepare_kernel, dim3(T), dim3(256), (size_t)(rot->dims + 2) * sizeof(float), resolve_stream(stream), cache, row, q, ldq, k, ldk, v, ldv,
-                       H * maps, G * maps, dn, G * dv, rot->freq, rot->mag, rot->dims, pos0);
+                       H * maps, G * maps, dn, G * dv, rot->freq, rot->mag, rot->dims, pos0, qb, kb, vb, temp_coef, temp_every);
     return last_launch_status();
 }
 
@@ -324,6 +342,8 @@ int ntk_window_attention(const ntk_window_attention_desc* d, void* stream) {
     a.pos0 = d->pos0; a.T = d->T; a.window = d->window; a.scale = d->scale; a.lambda = d->lambda; a.sub_norm = d->sub_norm; a.eps = d->eps; a.out_scale = d->out_scale;
     a.splits = d->scratch ? window_splits(d->T, d->H, d->G, window_keys(d->pos0, d->T, d->window)) : 1;
     a.scratch = d->scratch;
+    a.rel = d->rel; a.bucket_of = d->bucket_of; a.n_dist = d->n_dist;
+    if (a.rel && (!a.bucket_of || a.n_dist <= 0)) return NTK_E_NULL;
     const int DNP = (d->dn + 3) & ~3;
     const size_t lds = ((size_t)WROWS * d->maps * DNP + WKCH * (WSLAB + 1) + (size_t)d->maps * WROWS * WKCH) * sizeof(float);
     if (lds > 150 * 1024) return NTK_E_SHAPE;
