@@ -19,7 +19,7 @@ class DenseDesc(C.Structure):
     _fields_ = [("Y", C.c_void_p), ("ldy", C.c_int), ("X", C.c_void_p), ("ldx", C.c_int), ("W", C.c_void_p), ("wstride", C.c_longlong), ("wdtype", C.c_int),
                 ("offsets", C.c_void_p), ("G", C.c_int), ("rows", C.c_void_p), ("row_div", C.c_int), ("T", C.c_int), ("N", C.c_int), ("K", C.c_int),
                 ("accumulate", C.c_int), ("glu_ff", C.c_int), ("glu_limit", C.c_float), ("glu_alpha", C.c_float),
-                ("norm_w", C.c_void_p), ("norm_eps", C.c_float), ("norm_offset", C.c_float), ("glu_up_offset", C.c_float)]
+                ("norm_w", C.c_void_p), ("norm_eps", C.c_float), ("norm_offset", C.c_float), ("glu_up_offset", C.c_float), ("glu_cubic", C.c_float)]
 
 
 class Rotary(C.Structure):
@@ -29,7 +29,24 @@ class Rotary(C.Structure):
 class WindowAttentionDesc(C.Structure):
     _fields_ = [("out", C.c_void_p), ("ldo", C.c_int), ("q", C.c_void_p), ("ldq", C.c_int), ("cache", C.c_void_p), ("row", C.c_int),
                 ("H", C.c_int), ("G", C.c_int), ("maps", C.c_int), ("dn", C.c_int), ("dv", C.c_int), ("pos0", C.c_int), ("T", C.c_int), ("window", C.c_int),
-                ("scale", C.c_float), ("lam", C.c_float), ("sub_norm", C.c_int), ("eps", C.c_float), ("out_scale", C.c_float), ("scratch", C.c_void_p)]
+                ("scale", C.c_float), ("lam", C.c_float), ("sub_norm", C.c_int), ("eps", C.c_float), ("out_scale", C.c_float), ("scratch", C.c_void_p),
+                ("rel", C.c_void_p), ("bucket_of", C.c_void_p), ("n_dist", C.c_int)]
+
+
+class GatedSeamDesc(C.Structure):
+    _fields_ = [("x", C.c_void_p), ("ldx", C.c_int), ("y", C.c_void_p), ("ldy", C.c_int), ("yb", C.c_void_p), ("g", C.c_void_p), ("ldg", C.c_int), ("gb", C.c_void_p),
+                ("hist", C.c_void_p), ("hist_stride", C.c_longlong), ("n_hist", C.c_int), ("coef", C.c_void_p),
+                ("h", C.c_void_p), ("ldh", C.c_int), ("nw", C.c_void_p), ("nb", C.c_void_p), ("alpha", C.c_float), ("T", C.c_int), ("n", C.c_int)]
+
+
+class GatedRecurrenceDesc(C.Structure):
+    _fields_ = [("out", C.c_void_p), ("ldo", C.c_int), ("q", C.c_void_p), ("ldq", C.c_int), ("k", C.c_void_p), ("ldk", C.c_int), ("v", C.c_void_p), ("ldv", C.c_int),
+                ("wz", C.c_void_p), ("ldw", C.c_int), ("wb", C.c_void_p), ("decay_form", C.c_int), ("decay_param", C.c_float),
+                ("az", C.c_void_p), ("lda", C.c_int), ("ab", C.c_void_p), ("unit_eps", C.c_float), ("state", C.c_void_p),
+                ("H", C.c_int), ("dn", C.c_int), ("dv", C.c_int), ("q_scale", C.c_float), ("pos0", C.c_int), ("T", C.c_int)]
+
+
+DECAY_GIVEN, DECAY_SIGMOID_ROOT, DECAY_EXP_SIGMOID = 0, 1, 2
 
 
 class RouteDesc(C.Structure):
@@ -77,6 +94,15 @@ def _bind():
     L.ntk_moe_route_ex.argtypes = [vp, vp, vp, vp, i, vp, vp, i, i, i, i, C.POINTER(RouteDesc), vp]
     L.ntk_glu.argtypes = [vp, vp, i, i, f, f, f, vp]
     L.ntk_moe_sum.argtypes = [vp, vp, vp, vp, vp, vp, i, i, i, vp]
+    L.ntk_dyt.argtypes = [vp, i, vp, i, vp, vp, f, i, i, vp]
+    L.ntk_embed_positions.argtypes = [vp, vp, vp, vp, i, vp, i, i, i, i, i, vp, vp, f, vp]
+    L.ntk_sigmoid_gate_scaled.argtypes = [vp, i, vp, i, vp, f, i, i, vp]
+    L.ntk_tanh_rows.argtypes = [vp, i, i, i, vp]
+    L.ntk_head_rmsnorm_gate.argtypes = [vp, i, vp, i, vp, i, vp, i, i, f, i, i, i, f, vp]
+    L.ntk_gated_seam.argtypes = [C.POINTER(GatedSeamDesc), vp]
+    L.ntk_window_prepare_biased.argtypes = [vp, i, vp, i, vp, i, vp, i, i, i, i, i, i, C.POINTER(Rotary), vp, vp, vp, f, C.c_double, i, i, vp]
+    L.ntk_gated_recurrence.argtypes = [C.POINTER(GatedRecurrenceDesc), vp]
+    L.ntk_glu_cubic.argtypes = [vp, vp, i, i, i, f, f, f, f, vp]
     L._layers_bound = True
     return L
 
@@ -110,7 +136,7 @@ def _i(a) -> DeviceBuffer:
 
 def dense(x: np.ndarray, w: np.ndarray, dtype: str = "float32", offsets=None, rows=None, row_div: int = 1, n_rows: Optional[int] = None,
           y0: Optional[np.ndarray] = None, glu_limit: Optional[float] = None, glu_alpha: float = 1.702, norm_w: Optional[np.ndarray] = None,
-          norm_eps: float = 1e-6, norm_offset: float = 0.0, glu_up_offset: float = 1.0) -> np.ndarray:
+          norm_eps: float = 1e-6, norm_offset: float = 0.0, glu_up_offset: float = 1.0, glu_cubic: float = 0.0) -> np.ndarray:
     """y[r] = x[src(r)] . w[g(r)]^T; w [N, K] or a stack [G, N, K] with `offsets` [G + 1]; rows: source row per output row (divided by row_div);
     y0: start values to accumulate onto."""
     L = _bind()
@@ -123,7 +149,7 @@ def dense(x: np.ndarray, w: np.ndarray, dtype: str = "float32", offsets=None, ro
     ob = _i(offsets) if offsets is not None else None
     rb = _i(rows) if rows is not None else None
     d = DenseDesc(yb.ptr, N, xb.ptr, x.shape[1], wb.ptr, N * K if stacked else 0, wdt, ob.ptr if ob else None, w.shape[0] if stacked else 1,
-                  rb.ptr if rb else None, row_div, T, N, K, int(y0 is not None), 0, 0.0, 0.0, None, 0.0, 0.0, glu_up_offset)
+                  rb.ptr if rb else None, row_div, T, N, K, int(y0 is not None), 0, 0.0, 0.0, None, 0.0, 0.0, glu_up_offset, glu_cubic)
     nb = _f(norm_w) if norm_w is not None else None
     if nb is not None:          # fused RMS norm of the activation rows (few rows)
         d.norm_w, d.norm_eps, d.norm_offset = nb.ptr, norm_eps, norm_offset
@@ -319,16 +345,36 @@ def window_prepare(q: np.ndarray, k: np.ndarray, v: np.ndarray, H: int, G: int, 
     return cb.numpy(np.float32, n * row).reshape(n, row), qb.numpy(np.float32, q.size).reshape(q.shape)
 
 
+def window_prepare_biased(q, k, v, H: int, G: int, dn: int, dv: int, pos0: int, qb=None, kb=None, vb=None, temp_coef: float = 0.0, temp_every: float = 1.0,
+                          cache: Optional[np.ndarray] = None, cache_rows: Optional[int] = None):
+    """no rotation, one score map: q = (q + qb) * temperature(position), k + kb and v + vb into the cache rows -> (cache, q)"""
+    L = _bind()
+    T, row = q.shape[0], G * (dn + dv)
+    n = cache_rows or (pos0 + T)
+    cb = _f(cache) if cache is not None else DeviceBuffer.zeros(n * row * 4)
+    qd, kd, vd = _f(q), _f(k), _f(v)
+    bq, bk, bv = (_f(x) if x is not None else None for x in (qb, kb, vb))
+    rot = Rotary(None, 1.0, 0)
+    check(L.ntk_window_prepare_biased(cb.ptr, row, qd.ptr, q.shape[1], kd.ptr, k.shape[1], vd.ptr, v.shape[1], H, G, 1, dn, dv, C.byref(rot), bq.ptr if bq else None,
+                                      bk.ptr if bk else None, bv.ptr if bv else None, temp_coef, temp_every, pos0, T, None), "ntk_window_prepare_biased")
+    return cb.numpy(np.float32, n * row).reshape(n, row), qd.numpy(np.float32, q.size).reshape(q.shape)
+
+
 def window_attention(q: np.ndarray, cache: np.ndarray, H: int, G: int, maps: int, dn: int, dv: int, pos0: int, window: int, scale: float, lam: float = 0.0,
-                     sub_norm: bool = False, eps: float = 1e-6, out_scale: float = 1.0, split: bool = True) -> np.ndarray:
-    """q [T, H * maps * dn] (rotated), cache rows [G][maps][dn] keys | [G][dv] values; split: long key ranges of few rows may be cut into merged parts"""
+                     sub_norm: bool = False, eps: float = 1e-6, out_scale: float = 1.0, split: bool = True, rel: Optional[np.ndarray] = None,
+                     bucket_of: Optional[np.ndarray] = None) -> np.ndarray:
+    """q [T, H * maps * dn] (rotated), cache rows [G][maps][dn] keys | [G][dv] values; split: long key ranges of few rows may be cut into merged parts;
+    rel [buckets, H] with bucket_of [distances]: a bias by distance on the scaled score"""
     L = _bind()
     T, row = q.shape[0], G * (maps * dn + dv)
     qb, cb = _f(q), _f(cache)
     out = DeviceBuffer.zeros(T * H * dv * 4)
     sc = DeviceBuffer.zeros(max(int(L.ntk_window_attention_scratch(T, H, maps, dv, pos0 + T)), 1) * 4) if split else None
     d = WindowAttentionDesc(out.ptr, H * dv, qb.ptr, q.shape[1], cb.ptr, row, H, G, maps, dn, dv, pos0, T, window, scale, lam, int(sub_norm), eps, out_scale,
-                            sc.ptr if sc else None)
+                            sc.ptr if sc else None, None, None, 0)
+    if rel is not None:
+        rb, bb = _f(rel), _i(bucket_of)
+        d.rel, d.bucket_of, d.n_dist = rb.ptr, bb.ptr, len(bucket_of)
     check(L.ntk_window_attention(C.byref(d), None), "ntk_window_attention")
     return out.numpy(np.float32, T * H * dv).reshape(T, H * dv)
 
@@ -382,3 +428,90 @@ def moe_sum(d, where, wts, shared=None, sgate=None) -> np.ndarray:
     out = DeviceBuffer.zeros(T * n * 4)
     check(L.ntk_moe_sum(out.ptr, db.ptr, wb.ptr, tb.ptr, sb.ptr if sb else None, gb.ptr if gb else None, T, top, n, None), "ntk_moe_sum")
     return out.numpy(np.float32, T * n).reshape(T, n)
+
+
+def dyt(x: np.ndarray, w: np.ndarray, b: Optional[np.ndarray], alpha: float) -> np.ndarray:
+    L = _bind()
+    T, n = x.shape
+    xb, wb = _f(x), _f(w)
+    bb = _f(b) if b is not None else None
+    out = DeviceBuffer.zeros(T * n * 4)
+    check(L.ntk_dyt(out.ptr, n, xb.ptr, n, wb.ptr, bb.ptr if bb else None, alpha, T, n, None), "ntk_dyt")
+    return out.numpy(np.float32, T * n).reshape(T, n)
+
+
+def embed_positions(table: np.ndarray, pos_table: np.ndarray, tokens, pos0: int, w=None, b=None, alpha: float = 0.0, dtype: str = "float32") -> np.ndarray:
+    L = _bind()
+    T, (V, W) = len(tokens), table.shape
+    (tb, dt), (pb, _) = weight_buffer(table, dtype), weight_buffer(pos_table, dtype)
+    ib = _i(tokens)
+    wb, bb = (_f(x) if x is not None else None for x in (w, b))
+    out = DeviceBuffer.zeros(T * W * 4)
+    check(L.ntk_embed_positions(out.ptr, None, tb.ptr, pb.ptr, dt, ib.ptr, T, V, W, pos0, pos_table.shape[0], wb.ptr if wb else None, bb.ptr if bb else None, alpha,
+                                None), "ntk_embed_positions")
+    return out.numpy(np.float32, T * W).reshape(T, W)
+
+
+def sigmoid_gate_scaled(y: np.ndarray, g: np.ndarray, gb=None, scale: float = 1.0) -> np.ndarray:
+    L = _bind()
+    T, n = y.shape
+    yb, gd = _f(y), _f(g)
+    bb = _f(gb) if gb is not None else None
+    check(L.ntk_sigmoid_gate_scaled(yb.ptr, n, gd.ptr, n, bb.ptr if bb else None, scale, T, n, None), "ntk_sigmoid_gate_scaled")
+    return yb.numpy(np.float32, T * n).reshape(T, n)
+
+
+def head_rmsnorm_gate(x: np.ndarray, w: np.ndarray, H: int, dv: int, eps: float, g=None, act: int = 0, scale: float = 1.0, per_head: bool = False) -> np.ndarray:
+    """w [dv] (shared by the heads) or, per_head, [H * dv]; act 0 none, 1 sigmoid(g), 2 silu(g)"""
+    L = _bind()
+    T = x.shape[0]
+    xb, wb = _f(x), _f(w)
+    gb = _f(g) if g is not None else None
+    out = DeviceBuffer.zeros(T * H * dv * 4)
+    check(L.ntk_head_rmsnorm_gate(out.ptr, H * dv, xb.ptr, H * dv, wb.ptr, dv if per_head else 0, gb.ptr if gb else None, H * dv, act,
+                                  scale, T, H, dv, eps, None), "ntk_head_rmsnorm_gate")
+    return out.numpy(np.float32, T * H * dv).reshape(T, H * dv)
+
+
+def gated_seam(x, y=None, g=None, yb=None, gb=None, hist=None, coef=None, norm=None):
+    """x [T, n] stream, y / g a sublayer's result and gate pre-activations; hist [n_hist, T, n] (its last entry is overwritten with the new layer result) with
+    coef [n_hist]; norm = (w, b, alpha) -> (x, hist, h)"""
+    L = _bind()
+    T, n = x.shape
+    xb = _f(x)
+    bufs = {k: (_f(v) if v is not None else None) for k, v in dict(y=y, g=g, yb=yb, gb=gb, hist=hist, coef=coef).items()}
+    p = lambda k: bufs[k].ptr if bufs[k] else None
+    hb = DeviceBuffer.zeros(T * n * 4) if norm is not None else None
+    nw, nb = (_f(norm[0]), _f(norm[1])) if norm is not None else (None, None)
+    d = GatedSeamDesc(xb.ptr, n, p("y"), n, p("yb"), p("g"), n, p("gb"), p("hist"), T * n, 0 if hist is None else hist.shape[0], p("coef"),
+                      hb.ptr if hb else None, n, nw.ptr if nw else None, nb.ptr if nb else None, norm[2] if norm is not None else 0.0, T, n)
+    check(L.ntk_gated_seam(C.byref(d), None), "ntk_gated_seam")
+    return (xb.numpy(np.float32, T * n).reshape(T, n), bufs["hist"].numpy(np.float32, hist.size).reshape(hist.shape) if hist is not None else None,
+            hb.numpy(np.float32, T * n).reshape(T, n) if hb else None)
+
+
+def gated_recurrence(q, k, v, wz, H: int, dn: int, dv: int, pos0: int, decay_form: int = DECAY_GIVEN, decay_param: float = 1.0, wb=None, az=None, ab=None,
+                     unit_eps: float = 1e-6, q_scale: float = 1.0, state: Optional[np.ndarray] = None):
+    """-> (out [T, H * dv], state [H, dn, dv]); az: the removal rate's raw projection (None: no removal term); state: what an earlier portion left (ignored when
+    pos0 == 0; by default full of NaN so that a read at the start would show)"""
+    L = _bind()
+    T = q.shape[0]
+    qb, kb, vb, zb = _f(q), _f(k), _f(v), _f(wz)
+    wbb, azb, abb = (_f(x) if x is not None else None for x in (wb, az, ab))
+    sb = _f(state) if state is not None else DeviceBuffer.from_numpy(np.full(H * dn * dv, np.nan, np.float32))
+    out = DeviceBuffer.zeros(T * H * dv * 4)
+    d = GatedRecurrenceDesc(out.ptr, H * dv, qb.ptr, q.shape[1], kb.ptr, k.shape[1], vb.ptr, v.shape[1], zb.ptr, wz.shape[1], wbb.ptr if wbb else None, decay_form,
+                            decay_param, azb.ptr if azb else None, az.shape[1] if az is not None else 0, abb.ptr if abb else None, unit_eps, sb.ptr, H, dn, dv, q_scale,
+                            pos0, T)
+    check(L.ntk_gated_recurrence(C.byref(d), None), "ntk_gated_recurrence")
+    return out.numpy(np.float32, T * H * dv).reshape(T, H * dv), sb.numpy(np.float32, H * dn * dv).reshape(H, dn, dv)
+
+
+def glu_cubic(gu: np.ndarray, ff: int, alpha: float, cubic: float, limit: float = float("inf"), up_offset: float = 0.0) -> np.ndarray:
+    """gu rows may be longer than 2 * ff (what lies behind the up values is ignored)"""
+    L = _bind()
+    rows = gu.shape[0]
+    gb = _f(gu)
+    out = DeviceBuffer.zeros(rows * ff * 4)
+    check(L.ntk_glu_cubic(out.ptr, gb.ptr, gu.shape[1], rows, ff, limit, alpha, cubic, up_offset, None), "ntk_glu_cubic")
+    return out.numpy(np.float32, rows * ff).reshape(rows, ff)

@@ -68,10 +68,10 @@ def fabolorn_shapes(cfg: dict) -> Dict[str, Tuple[int, ...]]:
     return s
 
 
-def nizorax_config(preset: str, layers: int = 2) -> dict:
+def nizorax_config(preset: str, layers: int = 2, dense_only: bool = False) -> dict:
     """the sequential family at the preset's width, heads, experts and vocabulary: attention layers (two score maps of half the preset's key size each,
-    four query heads per key/value head, the preset's window) alternate with lightning layers; every third layer has the dense feed-forward at the
-    mixture's active width, the others the mixture (groups of eight experts, half of the groups open)"""
+    four query heads per key/value head, the preset's window) alternate with lightning layers; every third layer (dense_only: every layer) has the dense
+    feed-forward at the mixture's active width, the others the mixture (groups of eight experts, half of the groups open)"""
     p = PRESETS[preset]
     H, dn = p["heads"], p["dim"] + p["rot_dim"]
     ls = []
@@ -83,7 +83,7 @@ def nizorax_config(preset: str, layers: int = 2) -> dict:
         else:
             mx = {"heads": H, "dim": dn // 2 if dn // 2 <= 128 else 128, "vdim": p["vdim"], "decay": [1.0 - 2.0 ** (-5.0 - 3.0 * h / max(H - 1, 1)) for h in range(H)]}
             t = "lightning"
-        if k % 3 == 2:
+        if k % 3 == 2 or dense_only:
             ml = {"kind": "dense", "ff": p["top"] * p["ff"] + p["shared_ff"]}
         else:
             per = 8 if p["experts"] % 8 == 0 and p["experts"] >= 16 else 1
@@ -128,8 +128,60 @@ def nizorax_shapes(cfg: dict) -> Dict[str, Tuple[int, ...]]:
     return s
 
 
+def tubazen_config(preset: str, layers: int = 2, positions: int = 8192) -> dict:
+    """the gated family at the preset's width, heads and vocabulary: layers with two mixers side by side (attention over four query heads per key/value
+    head with a distance-bias table of 32 rows, beside a delta-rule recurrence with 64-entry keys) alternate with gated-linear-attention layers (keys 96,
+    the preset's value size); every layer has the gated feed-forward with the bytes of a two-matrix feed-forward at the mixture's active width"""
+    p = PRESETS[preset]
+    H, dn = p["heads"], p["dim"]
+    ff = (p["top"] * p["ff"] + p["shared_ff"]) * 2 // 3
+    ff -= ff % 64
+    ls = []
+    for k in range(layers):
+        if k % 2 == 0:
+            left = {"heads": H, "kv_heads": max(H // 4, 1), "dim": dn, "vdim": p["vdim"], "bias_max": 4096, "scale": 1.0 / math.sqrt(dn), "q_temp": {"coef": 0.1, "every": 512}}
+            mx = {"left": left, "right": {"heads": H, "dim": max(dn // 2, 8)}, "left_scale": 0.8, "right_scale": 0.5}
+            t = "parallel"
+        else:
+            mx = {"heads": H, "dim": max(3 * dn // 4, 8), "vdim": p["vdim"], "tau": 16.0}
+            t = "gla"
+        ls.append({"type": t, "mixer": mx, "mlp": {"kind": "dense", "ff": max(ff, 64)}})
+    return {"architecture": "Tubazen", "layers": ls, "norm": {"eps": 1e-5}, "logit_scale": 1.0 / math.sqrt(p["width"]), "max_positions": positions,
+            "vocab": p["vocab"], "width": p["width"]}
+
+
+def tubazen_shapes(cfg: dict, buckets: int = 32, rank: int = 64) -> Dict[str, Tuple[int, ...]]:
+    W, V = cfg["width"], cfg["vocab"]
+    rank = min(rank, max(W // 8, 4))
+    s: Dict[str, Tuple[int, ...]] = {"embed": (V, W), "pos": (cfg["max_positions"], W), "head": (V, W)}
+    for nm in ("embed.norm", "final.norm"):
+        s[nm], s[nm + ".b"], s[nm + ".alpha"] = (W,), (W,), ()
+    for i, L in enumerate(cfg["layers"]):
+        p, mx, ml = "l%d." % i, L["mixer"], L.get("mlp")
+        for nm in ("norm1",) + (("norm2",) if ml else ()):
+            s[p + nm], s[p + nm + ".b"], s[p + nm + ".alpha"] = (W,), (W,), ()
+        s[p + "rg1"], s[p + "rg1.b"], s[p + "dwa"] = (W, W), (W,), (i + 2,)
+        if L["type"] == "gla":
+            H, dn, dv, q = mx["heads"], mx["dim"], mx["vdim"], p + "mix."
+            s[q + "q"], s[q + "k"], s[q + "v"], s[q + "g"], s[q + "o"], s[q + "norm"] = (H * dn, W), (H * dn, W), (H * dv, W), (H * dv, W), (W, H * dv), (dv,)
+            s[q + "a1"], s[q + "a2"], s[q + "a2.b"] = (rank, W), (H * dn, rank), (H * dn,)
+        else:
+            l, r = mx["left"], mx["right"]
+            H, G, dn, dv, q = l["heads"], l.get("kv_heads", l["heads"]), l["dim"], l["vdim"], p + "mix.left."
+            s[q + "q"], s[q + "q.b"], s[q + "k"], s[q + "k.b"], s[q + "v"], s[q + "v.b"] = (H * dn, W), (H * dn,), (G * dn, W), (G * dn,), (G * dv, W), (G * dv,)
+            s[q + "rel"], s[q + "g"], s[q + "o"], s[q + "o.b"] = (buckets, H), (H * dv, W), (W, H * dv), (W,)
+            q, hd = p + "mix.right.", r["heads"] * r["dim"]
+            for nm in ("r", "k", "v", "g", "a"):
+                s[q + nm] = (hd, W)
+            s[q + "a.b"], s[q + "w1"], s[q + "w2"], s[q + "w0"], s[q + "norm"], s[q + "o"] = (hd,), (rank, W), (hd, rank), (hd,), (hd,), (W, hd)
+        if ml:
+            s[p + "mlp.gate"], s[p + "mlp.up"], s[p + "mlp.down"], s[p + "rg2"], s[p + "rg2.b"] = (ml["ff"], W), (ml["ff"], W), (W, ml["ff"]), (W, W), (W,)
+    return s
+
+
 def shapes_of(cfg: dict) -> Dict[str, Tuple[int, ...]]:
-    return nizorax_shapes(cfg) if cfg.get("architecture") == "Nizorax" else fabolorn_shapes(cfg)
+    arch = cfg.get("architecture")
+    return nizorax_shapes(cfg) if arch == "Nizorax" else tubazen_shapes(cfg) if arch == "Tubazen" else fabolorn_shapes(cfg)
 
 
 def _bf16(a: np.ndarray) -> np.ndarray:
@@ -157,8 +209,14 @@ def write_folder(folder: str, cfg: dict, seed: int = 20260925) -> int:
         f.write(hj)
         for k, (name, shp) in enumerate(shapes.items()):
             n = int(np.prod(shp))
+            if len(shp) == 0 or name.endswith(".dwa"):       # a norm's slope around one; depth weights: an average over the results so far
+                vals = (1.0 + 0.1 * pool[:1]) if len(shp) == 0 else (1.0 / n + 0.01 * pool[:n])
+                f.write(_bf16(vals).tobytes())
+                continue
             if len(shp) == 1:
                 around_one = name.endswith(".norm") and name != "final.norm"
+                if cfg.get("architecture") == "Tubazen":
+                    around_one = name.rsplit(".", 1)[-1] in ("norm", "norm1", "norm2")
                 if cfg.get("architecture") == "Nizorax":     # layer-norm weights around one, biases / lambda vectors / activation numbers small
                     around_one = name.rsplit(".", 1)[-1] in ("norm", "norm1", "norm2", "norm1b", "norm2b")
                 vals = 0.1 * pool[:n] + (1.0 if around_one else 0.0)
