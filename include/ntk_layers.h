@@ -227,7 +227,10 @@ typedef struct ntk_gated_recurrence_desc {
     int H, dn, dv;
     float q_scale;
     int pos0, T;
+    float* scratch;   /* F32 [>= ntk_gated_recurrence_scratch(T, H, dn, az != NULL)]: portions of more than a few tokens form their per-token vectors in a launch
+                         of their own, once per head instead of once per workgroup; NULL: always inside the walk */
 } ntk_gated_recurrence_desc;
+size_t ntk_gated_recurrence_scratch(int T, int H, int dn, int removal);
 int ntk_gated_recurrence(const ntk_gated_recurrence_desc* d, void* stream);
 
 /* ---- moe.hip ---------------------------------------------------------------------------------------------------------------------- */

@@ -664,7 +664,7 @@ int LayerStackModel::load(const std::string& dir, const SeqLoadOptions& opt) {
 int LayerStackModel::alloc_buffers() {
     const int W = info_.width;
     chunk_ = std::min(opt_.max_context, 1024);
-    size_t sc = 0, wsc = 0, lsc = 0;
+    size_t sc = 0, wsc = 0, lsc = 0, rsc = 0;
     for (const auto& L : layers_) {
         if (L.mixer == kMixLatent) {
             const LatentMixer& m = L.mix;
@@ -693,11 +693,13 @@ int LayerStackModel::alloc_buffers() {
             max_in_ = std::max<int>(max_in_, (int)m.in.out_f);
             max_hdv_ = std::max(max_hdv_, m.heads * m.vdim);
             max_rec_ = std::max(max_rec_, m.heads * m.dim);
+            rsc = std::max(rsc, ntk_gated_recurrence_scratch(chunk_, m.heads, m.dim, 0));
         } else {
             const ParallelMixer& m = L.par;
             max_in_ = std::max<int>(max_in_, (int)m.in.out_f);
             max_hdv_ = std::max<int>(max_hdv_, (int)m.o.in_f);
             max_rec_ = std::max(max_rec_, m.right.heads * m.right.dim);
+            rsc = std::max(rsc, ntk_gated_recurrence_scratch(chunk_, m.right.heads, m.right.dim, 1));
             wsc = std::max(wsc, ntk_window_attention_scratch(chunk_, m.left.heads, 1, m.left.vdim, opt_.max_context));
         }
         if (form_.gated && L.has_mlp) max_gu2_ = std::max<int>(max_gu2_, (int)L.gff.in.out_f), max_ffn_ = std::max(max_ffn_, L.gff.ff);
@@ -720,7 +722,7 @@ int LayerStackModel::alloc_buffers() {
              fl(&lat_, (size_t)kSharedRows * max_hr_) && fl(&kx_, ctx * max_hdn_) && fl(&vx_, ctx * max_hdv_) && fl(&scratch_, sc);
     if (form_.sequential) ok = ok && fl(&hist_, (C + (size_t)taps_ - 1) * W) && fl(&ff_, C * W) && fl(&zf_, C * max_ffn_) && fl(&wscratch_, wsc) && fl(&lscratch_, lsc);
     if (form_.gated)
-        ok = ok && fl(&ff_, C * W) && fl(&zf_, C * max_ffn_) && fl(&wscratch_, wsc) && fl(&results_, (runs_.size() + 1) * C * W) && fl(&zq_, C * std::max(max_rec_, 1)) &&
+        ok = ok && fl(&ff_, C * W) && fl(&zf_, C * max_ffn_) && fl(&wscratch_, wsc) && fl(&results_, (runs_.size() + 1) * C * W) && fl(&zq_, C * std::max(max_rec_, 1)) && fl(&rscratch_, rsc) &&
              fl(&gu2_, C * std::max(max_gu2_, 1));
     want_dev_ = tokens_dev_ ? tokens_dev_ + C : nullptr;   // one staging area: [tokens of a pass | wanted places], filled by ONE stream-ordered copy from pinned memory
     h_stage_ = (int*)nt_hip_malloc_host(2 * C * sizeof(int));
@@ -879,7 +881,7 @@ int LayerStackModel::run_gla(const StackLayer& L, float* state, int T, int pos0)
     ntk_gated_recurrence_desc d{};
     d.out = att_; d.ldo = hv; d.q = a_; d.ldq = na; d.k = a_ + m.k_off; d.ldk = na; d.v = a_ + m.v_off; d.ldv = na;
     d.wz = zq_; d.ldw = hq; d.wb = m.a2_b; d.decay_form = NTK_DECAY_SIGMOID_ROOT; d.decay_param = m.tau;
-    d.state = state; d.H = m.heads; d.dn = m.dim; d.dv = m.vdim; d.q_scale = 1.0f / std::sqrt((float)m.dim); d.pos0 = pos0; d.T = T;
+    d.state = state; d.H = m.heads; d.dn = m.dim; d.dv = m.vdim; d.q_scale = 1.0f / std::sqrt((float)m.dim); d.pos0 = pos0; d.T = T; d.scratch = rscratch_;
     LS_TRY(ntk_gated_recurrence(&d, stream_));
     LS_TRY(ntk_head_rmsnorm_gate(att_, hv, att_, hv, m.norm, 0, a_ + m.g_off, na, 2, 1.0f, T, m.heads, m.vdim, eps_, stream_));
     return ntk_dense_linear(mix_, W, att_, hv, m.o.ptr, m.o.dtype, T, W, hv, 0, stream_);
@@ -911,7 +913,7 @@ int LayerStackModel::run_parallel(const StackLayer& L, float* cache, float* stat
     g.out = att_ + hv; g.ldo = no; g.q = a_ + r.r_off; g.ldq = na; g.k = a_ + r.k_off; g.ldk = na; g.v = a_ + r.v_off; g.ldv = na;
     g.wz = zq_; g.ldw = hd; g.wb = r.w0; g.decay_form = NTK_DECAY_EXP_SIGMOID; g.decay_param = kDeltaDecayRate;
     g.az = a_ + r.a_off; g.lda = na; g.ab = r.a_b; g.unit_eps = kUnitKeyEps;
-    g.state = state; g.H = r.heads; g.dn = r.dim; g.dv = r.dim; g.q_scale = 1.0f; g.pos0 = pos0; g.T = T;
+    g.state = state; g.H = r.heads; g.dn = r.dim; g.dv = r.dim; g.q_scale = 1.0f; g.pos0 = pos0; g.T = T; g.scratch = rscratch_;
     LS_TRY(ntk_gated_recurrence(&g, stream_));
     LS_TRY(ntk_head_rmsnorm_gate(att_ + hv, no, att_ + hv, no, r.norm, r.dim, a_ + r.g_off, na, 1, m.right_scale, T, r.heads, r.dim, eps_, stream_));
     return ntk_dense_linear(mix_, W, att_, no, m.o.ptr, m.o.dtype, T, W, no, 0, stream_);

@@ -276,7 +276,7 @@ private:
     float *x_ = nullptr, *x0_ = nullptr, *cat_ = nullptr, *h1_ = nullptr, *h2_ = nullptr, *a_ = nullptr, *cq_ = nullptr, *q_ = nullptr, *qf_ = nullptr, *lat_ = nullptr,
           *att_ = nullptr, *kx_ = nullptr, *vx_ = nullptr, *mix_ = nullptr, *wts_ = nullptr, *sg_ = nullptr, *gu_ = nullptr, *act_ = nullptr, *dn_ = nullptr,
           *sgu_ = nullptr, *sact_ = nullptr, *sdn_ = nullptr, *scratch_ = nullptr, *xw_ = nullptr, *hn_ = nullptr, *hist_ = nullptr, *ff_ = nullptr, *zf_ = nullptr, *wscratch_ = nullptr, *lscratch_ = nullptr,
-          *results_ = nullptr, *zq_ = nullptr, *gu2_ = nullptr;   // gated form: the layer results of the pass [runs + 1][chunk][width], decay pre-activations, [gate | up | residual gate]
+          *results_ = nullptr, *zq_ = nullptr, *gu2_ = nullptr, *rscratch_ = nullptr;   // gated form: the layer results of the pass [runs + 1][chunk][width], decay pre-activations, [gate | up | residual gate]
     int max_rec_ = 0, max_gu2_ = 0;
     int *ids_ = nullptr, *offsets_ = nullptr, *order_ = nullptr, *where_ = nullptr, *tokens_dev_ = nullptr, *want_dev_ = nullptr;
     int* h_stage_ = nullptr;          // pinned: tokens and wanted places of the pass being launched

@@ -5,11 +5,14 @@
 // (the removal is taken from S_(t-1) as it was, not from the decayed state).  Without the removal term this is gated linear attention.  Everything behind the projections is F32.
 //
 // A column of the state never meets another column: u^T S, the update and S^T q are sums over key channels only.  So a lane owns RP rows of ONE value
-// column, SPLIT lanes next to each other share a column (their partial sums meet in a DPP reduction, twice per token with the removal term, once without),
+// column, SPLIT lanes next to each other share a column (their partial sums meet in a DPP reduction, twice per token with the removal term, once without;
+// only the first of the two lies on the chain from one token to the next),
 // and a wave walks the tokens in order without ever waiting for another wave: no barrier per token, the state stays in registers for the whole portion
 // and crosses HBM once in and once out.  The four waves of a workgroup share one head, so the per-token vectors -- q, k, the decay formed from its raw
 // projection, the removal rate times the unit key -- are staged for all of them in LDS, a batch of tokens at a time; the NEXT batch's raw values are
 // requested into registers before the current batch is walked, so their latency hides behind the walk.
+// Portions of more than a few tokens run a pre-pass first (one wave per token and head, the whole chip at once) that leaves those vectors ready-made in a
+// packed buffer [T][H][vectors][dn]: the walk's staging is then a copy, and what a head's workgroups would each have recomputed is computed once.
 // The walk is the same whatever the portion: a sequence cut anywhere gives the same sums in the same order.
 #include <algorithm>
 #include "common.hip.h"
@@ -28,9 +31,12 @@ struct RecArgs {
     int H, dn, dv;
     float q_scale;
     int pos0, T, TB;
+    float* packed;                   // [T][H][NV][dn] ready-made vectors (q * scale, k, w (, u, a * u)), or NULL: formed while staging
 };
 
-constexpr int REC_PF = 8;        // staged (token, channel) entries a thread carries from one batch to the next: TB * SPLIT * RP <= 256 * REC_PF
+constexpr int kRecFewTokens = 8;  // up to this many tokens (decoding) the walk forms its vectors itself: one launch
+// staged (token, channel) entries a thread carries from one batch to the next: TB * SPLIT * RP <= threads * rec_pf
+constexpr int rec_pf(int waves) { return waves == 1 ? 16 : 8; }
 
 __device__ __forceinline__ float decay_of(float z, int form, float param) {
     if (form == NTK_DECAY_SIGMOID_ROOT) {
@@ -42,15 +48,49 @@ __device__ __forceinline__ float decay_of(float z, int form, float param) {
     return z;
 }
 
-template <int SPLIT, int RP, bool DELTA>
-__global__ __launch_bounds__(256) void gated_recurrence_kernel(const RecArgs a) {
-    constexpr int CW = 64 / SPLIT, CB = 4 * CW;          // value columns per wave / per workgroup
+// the per-token vectors of one (token, head), ready for the walk: one wave each
+template <bool DELTA>
+__global__ __launch_bounds__(64) void gated_recurrence_prepare_kernel(const RecArgs a) {
+    constexpr int NV = DELTA ? 5 : 3;
+    const int lane = threadIdx.x, h = blockIdx.x % a.H;
+    const long long t = blockIdx.x / a.H;
+    float* dst = a.packed + (t * a.H + h) * NV * a.dn;
+    float ss = 0.0f;
+    for (int d = lane; d < a.dn; d += 64) {
+        const long long o = (long long)h * a.dn + d;
+        const float kk = a.k[t * a.ldk + o];
+        dst[d] = a.q[t * a.ldq + o] * a.q_scale;
+        dst[a.dn + d] = kk;
+        dst[2 * a.dn + d] = decay_of(a.wz[t * a.ldw + o] + (a.wb ? a.wb[o] : 0.0f), a.decay_form, a.decay_param);
+        ss = fmaf(kk, kk, ss);
+    }
+    if constexpr (DELTA) {
+        const float inv = 1.0f / sqrtf(wave_sum(ss) + a.unit_eps);      // (the same sum in the same lane order as the staging of the walk forms it)
+        for (int d = lane; d < a.dn; d += 64) {
+            const long long o = (long long)h * a.dn + d;
+            const float uu = a.k[t * a.ldk + o] * inv;
+            dst[3 * a.dn + d] = uu;
+            dst[4 * a.dn + d] = uu * (1.0f / (1.0f + expf(-(a.az[t * a.lda + o] + (a.ab ? a.ab[o] : 0.0f)))));
+        }
+    }
+}
+
+template <int RP, bool DELTA>
+struct TokVec {                      // one token's vectors as a lane needs them: its RP rows of q, k, w (, u, a * u) and its column's value
+    float q[RP], k[RP], w[RP], u[DELTA ? RP : 1], a[DELTA ? RP : 1], v;
+};
+
+template <int SPLIT, int RP, bool DELTA, bool PACKED, int NW>
+__global__ __launch_bounds__(64 * NW) void gated_recurrence_kernel(const RecArgs a) {
+    constexpr int NT = 64 * NW, REC_PF = rec_pf(NW);
+    constexpr int CW = 64 / SPLIT, CB = NW * CW;         // value columns per wave / per workgroup
     constexpr int RS = RP + 4;                           // LDS floats per lane group: the groups' 16-byte reads fall into different banks
     constexpr int DP = SPLIT * RP, DL = SPLIT * RS;      // key channels a workgroup covers (>= dn) / their LDS footprint
     constexpr int NV = DELTA ? 5 : 3;                    // staged vectors per token: q, k, w (, u, a * u)
     extern __shared__ __attribute__((aligned(16))) float lds[];
     float* Vec = lds;                                    // [TB][NV][DL]
-    float* Vs = lds + (size_t)a.TB * NV * DL;            // [TB][CB]
+    constexpr int EXTRA = RP <= 8 ? 2 : 0;               // token slots behind a batch (see the walk)
+    float* Vs = lds + (size_t)(a.TB + EXTRA) * NV * DL;  // [TB + EXTRA][CB]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int cl = lane / SPLIT, rg = lane % SPLIT;
     const int h = blockIdx.y, c0 = blockIdx.x * CB, c = c0 + wave * CW + cl;
@@ -63,14 +103,25 @@ __global__ __launch_bounds__(256) void gated_recurrence_kernel(const RecArgs a) 
         const int r = rg * RP + i;
         S[i] = (a.pos0 > 0 && col_ok && r < a.dn) ? st[(long long)r * a.dv] : 0.0f;
     }
+    // ---- the two slots behind a full batch: a token that leaves the state as it is and asks for nothing
+    for (int e = threadIdx.x; e < EXTRA * NV * DL; e += NT) Vec[(size_t)a.TB * NV * DL + e] = (e % (NV * DL)) / DL == 2 ? 1.0f : 0.0f;
+    for (int e = threadIdx.x; e < EXTRA * CB; e += NT) Vs[a.TB * CB + e] = 0.0f;
     // ---- raw values of a batch into registers (requests only), and from registers through the activations into LDS
-    float pq[REC_PF], pk[REC_PF], pw[REC_PF], pa[REC_PF], pv[2];
+    float pq[REC_PF], pk[REC_PF], pw[REC_PF], pa[REC_PF], pu[REC_PF], pv[2];
     auto request = [&](int t0, int nb) {
 #pragma unroll
         for (int u = 0; u < REC_PF; ++u) {
-            const int idx = threadIdx.x + 256 * u, tb = idx / DP, d = idx % DP;
+            const int idx = threadIdx.x + NT * u, tb = idx / DP, d = idx % DP;
             const bool ok = tb < nb && d < a.dn;
             const long long t = t0 + tb;
+            if constexpr (PACKED) {
+                const float* src = a.packed + ((t * a.H + h) * NV) * a.dn + d;
+                pq[u] = ok ? src[0] : 0.0f;
+                pk[u] = ok ? src[a.dn] : 0.0f;
+                pw[u] = ok ? src[2 * a.dn] : 1.0f;
+                if constexpr (DELTA) { pu[u] = ok ? src[3 * a.dn] : 0.0f; pa[u] = ok ? src[4 * a.dn] : 0.0f; }
+                continue;
+            }
             pq[u] = ok ? a.q[t * a.ldq + (long long)h * a.dn + d] : 0.0f;
             pk[u] = ok ? a.k[t * a.ldk + (long long)h * a.dn + d] : 0.0f;
             pw[u] = ok ? a.wz[t * a.ldw + (long long)h * a.dn + d] + (a.wb ? a.wb[h * a.dn + d] : 0.0f) : 0.0f;
@@ -78,30 +129,35 @@ __global__ __launch_bounds__(256) void gated_recurrence_kernel(const RecArgs a) 
         }
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            const int idx = threadIdx.x + 256 * u, tb = idx / CB, cc = idx % CB;
+            const int idx = threadIdx.x + NT * u, tb = idx / CB, cc = idx % CB;
             pv[u] = (tb < nb && c0 + cc < a.dv) ? a.v[(long long)(t0 + tb) * a.ldv + (long long)h * a.dv + c0 + cc] : 0.0f;
         }
     };
     auto stage = [&](int nb) {
 #pragma unroll
         for (int u = 0; u < REC_PF; ++u) {
-            const int idx = threadIdx.x + 256 * u, tb = idx / DP, d = idx % DP;
+            const int idx = threadIdx.x + NT * u, tb = idx / DP, d = idx % DP;
             if (tb >= a.TB) continue;
             const bool ok = tb < nb && d < a.dn;
             float* dst = Vec + (size_t)tb * NV * DL + (d / RP) * RS + d % RP;
+            if constexpr (PACKED) {
+                dst[0] = pq[u]; dst[DL] = pk[u]; dst[2 * DL] = pw[u];
+                if constexpr (DELTA) { dst[3 * DL] = pu[u]; dst[4 * DL] = pa[u]; }
+                continue;
+            }
             dst[0] = pq[u] * a.q_scale;
             dst[DL] = pk[u];
             dst[2 * DL] = ok ? decay_of(pw[u], a.decay_form, a.decay_param) : 1.0f;
-            if constexpr (DELTA) dst[4 * DL] = ok ? 1.0f / (1.0f + expf(-pa[u])) : 0.0f;     // the removal rate; times the unit key below
+            if constexpr (DELTA) { dst[3 * DL] = 0.0f; dst[4 * DL] = ok ? 1.0f / (1.0f + expf(-pa[u])) : 0.0f; }   // the removal rate; times the unit key below
         }
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            const int idx = threadIdx.x + 256 * u;
+            const int idx = threadIdx.x + NT * u;
             if (idx < a.TB * CB) Vs[idx] = pv[u];
         }
-        if constexpr (DELTA) {
+        if constexpr (DELTA && !PACKED) {
             __syncthreads();
-            for (int tb = wave; tb < nb; tb += 4) {      // a wave per token: the unit key (one sum over the head's channels, lanes in a fixed order)
+            for (int tb = wave; tb < nb; tb += NW) {     // a wave per token: the unit key (one sum over the head's channels, lanes in a fixed order)
                 float* base = Vec + (size_t)tb * NV * DL;
                 float ss = 0.0f;
                 for (int d = lane; d < a.dn; d += 64) { const float kk = base[DL + (d / RP) * RS + d % RP]; ss = fmaf(kk, kk, ss); }
@@ -122,40 +178,66 @@ __global__ __launch_bounds__(256) void gated_recurrence_kernel(const RecArgs a) 
         stage(nb);
         __syncthreads();
         if (t0 + a.TB < a.T) request(t0 + a.TB, min(a.TB, a.T - t0 - a.TB));
-        for (int tb = 0; tb < nb; ++tb) {
+        // The walk.  A token's vectors leave LDS one token AHEAD of their use (a second register set while the rows per lane are few), so the only chain from
+        // token to token is the state's own: u^T S, its reduction, the update.
+        auto load_tok = [&](int tb, TokVec<RP, DELTA>& x) {
             const float* base = Vec + (size_t)tb * NV * DL + rg * RS;
-            float qv[RP], kv[RP], wv[RP];
 #pragma unroll
             for (int i = 0; i < RP; i += 4) {
-                const float4 x = *reinterpret_cast<const float4*>(base + i), y = *reinterpret_cast<const float4*>(base + DL + i), z = *reinterpret_cast<const float4*>(base + 2 * DL + i);
-                qv[i] = x.x; qv[i + 1] = x.y; qv[i + 2] = x.z; qv[i + 3] = x.w;
-                kv[i] = y.x; kv[i + 1] = y.y; kv[i + 2] = y.z; kv[i + 3] = y.w;
-                wv[i] = z.x; wv[i + 1] = z.y; wv[i + 2] = z.z; wv[i + 3] = z.w;
-            }
-            const float vv = Vs[tb * CB + wave * CW + cl];
-            if constexpr (DELTA) {
-                float uv[RP], av[RP];
-#pragma unroll
-                for (int i = 0; i < RP; i += 4) {
-                    const float4 x = *reinterpret_cast<const float4*>(base + 3 * DL + i), y = *reinterpret_cast<const float4*>(base + 4 * DL + i);
-                    uv[i] = x.x; uv[i + 1] = x.y; uv[i + 2] = x.z; uv[i + 3] = x.w;
-                    av[i] = y.x; av[i + 1] = y.y; av[i + 2] = y.z; av[i + 3] = y.w;
+                const float4 q4 = *reinterpret_cast<const float4*>(base + i), k4 = *reinterpret_cast<const float4*>(base + DL + i), w4 = *reinterpret_cast<const float4*>(base + 2 * DL + i);
+                x.q[i] = q4.x; x.q[i + 1] = q4.y; x.q[i + 2] = q4.z; x.q[i + 3] = q4.w;
+                x.k[i] = k4.x; x.k[i + 1] = k4.y; x.k[i + 2] = k4.z; x.k[i + 3] = k4.w;
+                x.w[i] = w4.x; x.w[i + 1] = w4.y; x.w[i + 2] = w4.z; x.w[i + 3] = w4.w;
+                if constexpr (DELTA) {
+                    const float4 u4 = *reinterpret_cast<const float4*>(base + 3 * DL + i), a4 = *reinterpret_cast<const float4*>(base + 4 * DL + i);
+                    x.u[i] = u4.x; x.u[i + 1] = u4.y; x.u[i + 2] = u4.z; x.u[i + 3] = u4.w;
+                    x.a[i] = a4.x; x.a[i + 1] = a4.y; x.a[i + 2] = a4.z; x.a[i + 3] = a4.w;
                 }
-                float p = 0.0f;
+            }
+            x.v = Vs[tb * CB + wave * CW + cl];
+        };
+        // one token: the state's update, and the column's output as this lane's partial sum (the lanes' sums meet later, off the chain)
+        auto step = [&](const TokVec<RP, DELTA>& x) -> float {
+            if constexpr (DELTA) {
+                float p0 = 0.0f, p1 = 0.0f;              // (two partial sums: half the chain; rows in a fixed order either way)
 #pragma unroll
-                for (int i = 0; i < RP; ++i) p = fmaf(uv[i], S[i], p);
-                const float us = group_sum<SPLIT>(p);    // u^T S(t-1) of this column
+                for (int i = 0; i < RP; i += 2) { p0 = fmaf(x.u[i], S[i], p0); p1 = fmaf(x.u[i + 1], S[i + 1], p1); }
+                const float us = group_sum<SPLIT>(p0 + p1);   // u^T S(t-1) of this column
 #pragma unroll
-                for (int i = 0; i < RP; ++i) S[i] = fmaf(wv[i], S[i], fmaf(-av[i], us, kv[i] * vv));
+                for (int i = 0; i < RP; ++i) S[i] = fmaf(x.w[i], S[i], fmaf(-x.a[i], us, x.k[i] * x.v));
             } else {
 #pragma unroll
-                for (int i = 0; i < RP; ++i) S[i] = fmaf(wv[i], S[i], kv[i] * vv);
+                for (int i = 0; i < RP; ++i) S[i] = fmaf(x.w[i], S[i], x.k[i] * x.v);
             }
-            float o = 0.0f;
+            float o0 = 0.0f, o1 = 0.0f;
 #pragma unroll
-            for (int i = 0; i < RP; ++i) o = fmaf(S[i], qv[i], o);
-            o = group_sum<SPLIT>(o);
-            if (rg == 0 && col_ok) a.out[(long long)(t0 + tb) * a.ldo + (long long)h * a.dv + c] = o;
+            for (int i = 0; i < RP; i += 2) { o0 = fmaf(S[i], x.q[i], o0); o1 = fmaf(S[i + 1], x.q[i + 1], o1); }
+            return o0 + o1;
+        };
+        float* orow = a.out + (long long)t0 * a.ldo + (long long)h * a.dv + c;
+        if constexpr (RP <= 8) {
+            // two tokens per pass of the loop, no branch inside: the slots behind a batch's last token hold a token that changes nothing (decay one, the rest zero),
+            // so both register sets are always loaded and walked, and only the stores look at the token's number
+            TokVec<RP, DELTA> x0, x1;
+            load_tok(0, x0);
+            for (int tb = 0; tb < nb; tb += 2) {
+                load_tok(tb + 1, x1);
+                const float oa = step(x0);
+                load_tok(tb + 2, x0);
+                const float ob = step(x1);
+                const float ra = group_sum<SPLIT>(oa), rb = group_sum<SPLIT>(ob);
+                if (rg == 0 && col_ok) {
+                    orow[(long long)tb * a.ldo] = ra;
+                    if (tb + 1 < nb) orow[(long long)(tb + 1) * a.ldo] = rb;
+                }
+            }
+        } else {
+            for (int tb = 0; tb < nb; ++tb) {
+                TokVec<RP, DELTA> cur;
+                load_tok(tb, cur);
+                const float o = group_sum<SPLIT>(step(cur));
+                if (rg == 0 && col_ok) orow[(long long)tb * a.ldo] = o;
+            }
         }
     }
 #pragma unroll
@@ -165,28 +247,51 @@ __global__ __launch_bounds__(256) void gated_recurrence_kernel(const RecArgs a) 
     }
 }
 
-template <int SPLIT, int RP>
-static int launch_rec(const RecArgs& a0, hipStream_t s) {
+template <int SPLIT, int RP, int NW>
+static int launch_rec_waves(const RecArgs& a0, hipStream_t s) {
     RecArgs a = a0;
-    constexpr int CB = 4 * (64 / SPLIT), DP = SPLIT * RP, DL = SPLIT * (RP + 4);
+    constexpr int CB = NW * (64 / SPLIT), DP = SPLIT * RP, DL = SPLIT * (RP + 4), NT = 64 * NW;
     const bool delta = a.az != nullptr;
-    const int NV = delta ? 5 : 3;
-    int tb = (256 * REC_PF) / DP;                        // what a thread's registers carry
-    tb = std::min(tb, (2 * 256) / CB);                   // ... and of the values
+    const int NV = delta ? 5 : 3, extra = RP <= 8 ? 2 : 0;
+    int tb = (NT * rec_pf(NW)) / DP;                     // what a thread's registers carry
+    tb = std::min(tb, (2 * NT) / CB);                    // ... and of the values
     tb = std::min(tb, 16);
-    tb = std::min(tb, (int)(40 * 1024 / ((NV * DL + CB) * sizeof(float))));   // a batch's LDS stays under 40 KB: several workgroups per CU
+    tb = std::min(tb, (int)(40 * 1024 / ((NV * DL + CB) * sizeof(float))) - extra);   // a batch's LDS stays under 40 KB: several workgroups per CU
     tb = std::min(tb, std::max(a.T, 1));
     a.TB = std::max(tb, 1);
-    const size_t lds = ((size_t)a.TB * NV * DL + (size_t)a.TB * CB) * sizeof(float);
+    const size_t lds = (size_t)(a.TB + extra) * (NV * DL + CB) * sizeof(float);
     const dim3 grid((a.dv + CB - 1) / CB, a.H);
-    if (delta) hipLaunchKernelGGL((gated_recurrence_kernel<SPLIT, RP, true>), grid, dim3(256), lds, s, a);
-    else hipLaunchKernelGGL((gated_recurrence_kernel<SPLIT, RP, false>), grid, dim3(256), lds, s, a);
+    if (a.packed) {
+        if (delta) hipLaunchKernelGGL(gated_recurrence_prepare_kernel<true>, dim3(a.T * a.H), dim3(64), 0, s, a);
+        else hipLaunchKernelGGL(gated_recurrence_prepare_kernel<false>, dim3(a.T * a.H), dim3(64), 0, s, a);
+        const int st = last_launch_status();
+        if (st != NTK_OK) return st;
+        if (delta) hipLaunchKernelGGL((gated_recurrence_kernel<SPLIT, RP, true, true, NW>), grid, dim3(NT), lds, s, a);
+        else hipLaunchKernelGGL((gated_recurrence_kernel<SPLIT, RP, false, true, NW>), grid, dim3(NT), lds, s, a);
+        return last_launch_status();
+    }
+    if (delta) hipLaunchKernelGGL((gated_recurrence_kernel<SPLIT, RP, true, false, NW>), grid, dim3(NT), lds, s, a);
+    else hipLaunchKernelGGL((gated_recurrence_kernel<SPLIT, RP, false, false, NW>), grid, dim3(NT), lds, s, a);
     return last_launch_status();
+}
+
+// waves per workgroup: four share a head's staged vectors while that still leaves a workgroup per CU; fewer (down to one) where the columns are few, so
+// that the walk -- one chain per column, nothing to gain from a second wave on the same column -- spreads over the chip
+template <int SPLIT, int RP>
+static int launch_rec(const RecArgs& a, hipStream_t s) {
+    const long long col_groups = (long long)a.H * ((a.dv + 64 / SPLIT - 1) / (64 / SPLIT));   // waves of the launch
+    if (col_groups >= 4 * 256) return launch_rec_waves<SPLIT, RP, 4>(a, s);
+    if (col_groups >= 2 * 256) return launch_rec_waves<SPLIT, RP, 2>(a, s);
+    return launch_rec_waves<SPLIT, RP, 1>(a, s);
 }
 
 }  // namespace ntk
 
 using namespace ntk;
+
+size_t ntk_gated_recurrence_scratch(int T, int H, int dn, int removal) {
+    return T > kRecFewTokens ? (size_t)T * H * (removal ? 5 : 3) * dn : 0;
+}
 
 int ntk_gated_recurrence(const ntk_gated_recurrence_desc* d, void* stream) {
     if (!d || !d->out || !d->q || !d->k || !d->v || !d->wz || !d->state) return NTK_E_NULL;
@@ -197,20 +302,13 @@ int ntk_gated_recurrence(const ntk_gated_recurrence_desc* d, void* stream) {
     if (d->ldq < hd || d->ldk < hd || d->ldw < hd || (d->az && d->lda < hd) || d->ldv < d->H * d->dv || d->ldo < d->H * d->dv) return NTK_E_SHAPE;
     if (d->T == 0) return NTK_OK;
     RecArgs a{d->out, d->ldo, d->q, d->ldq, d->k, d->ldk, d->v, d->ldv, d->wz, d->ldw, d->wb, d->decay_form, d->decay_param, d->az, d->lda, d->ab, d->unit_eps,
-              d->state, d->H, d->dn, d->dv, d->q_scale, d->pos0, d->T, 0};
+              d->state, d->H, d->dn, d->dv, d->q_scale, d->pos0, d->T, 0, d->T > kRecFewTokens ? d->scratch : nullptr};
     hipStream_t s = resolve_stream(stream);
-    // Lanes per column: 32 (two columns per wave, 16 x the waves of the wide form) while the launch would otherwise leave most of the chip idle or the
-    // head's channels would not fit 8 lanes; rows per lane: the smallest of 4 / 8 / 16 / 32 that covers the channels.
-    const long long cols = (long long)d->H * d->dv;
-    const bool narrow = d->dn > 8 * 32 || cols / 8 < 2048;
-    if (narrow) {
-        if (d->dn <= 32 * 4) return launch_rec<32, 4>(a, s);
-        if (d->dn <= 32 * 8) return launch_rec<32, 8>(a, s);
-        if (d->dn <= 32 * 16) return launch_rec<32, 16>(a, s);
-        return launch_rec<32, 32>(a, s);
-    }
-    if (d->dn <= 8 * 4) return launch_rec<8, 4>(a, s);
-    if (d->dn <= 8 * 8) return launch_rec<8, 8>(a, s);
-    if (d->dn <= 8 * 16) return launch_rec<8, 16>(a, s);
-    return launch_rec<8, 32>(a, s);
+    // 16 lanes share a column (their sums meet in DPP steps inside a 16-lane row, no trip through LDS on the chain from token to token); rows per lane: the
+    // smallest of 4 / 8 / 16 / 32 that covers the head's channels; beyond 512 channels 32 lanes per column.
+    if (d->dn <= 16 * 4) return launch_rec<16, 4>(a, s);
+    if (d->dn <= 16 * 8) return launch_rec<16, 8>(a, s);
+    if (d->dn <= 16 * 16) return launch_rec<16, 16>(a, s);
+    if (d->dn <= 16 * 32) return launch_rec<16, 32>(a, s);
+    return launch_rec<32, 32>(a, s);
 }

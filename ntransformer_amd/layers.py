@@ -43,7 +43,7 @@ class GatedRecurrenceDesc(C.Structure):
     _fields_ = [("out", C.c_void_p), ("ldo", C.c_int), ("q", C.c_void_p), ("ldq", C.c_int), ("k", C.c_void_p), ("ldk", C.c_int), ("v", C.c_void_p), ("ldv", C.c_int),
                 ("wz", C.c_void_p), ("ldw", C.c_int), ("wb", C.c_void_p), ("decay_form", C.c_int), ("decay_param", C.c_float),
                 ("az", C.c_void_p), ("lda", C.c_int), ("ab", C.c_void_p), ("unit_eps", C.c_float), ("state", C.c_void_p),
-                ("H", C.c_int), ("dn", C.c_int), ("dv", C.c_int), ("q_scale", C.c_float), ("pos0", C.c_int), ("T", C.c_int)]
+                ("H", C.c_int), ("dn", C.c_int), ("dv", C.c_int), ("q_scale", C.c_float), ("pos0", C.c_int), ("T", C.c_int), ("scratch", C.c_void_p)]
 
 
 DECAY_GIVEN, DECAY_SIGMOID_ROOT, DECAY_EXP_SIGMOID = 0, 1, 2
@@ -102,6 +102,8 @@ def _bind():
     L.ntk_gated_seam.argtypes = [C.POINTER(GatedSeamDesc), vp]
     L.ntk_window_prepare_biased.argtypes = [vp, i, vp, i, vp, i, vp, i, i, i, i, i, i, C.POINTER(Rotary), vp, vp, vp, f, C.c_double, i, i, vp]
     L.ntk_gated_recurrence.argtypes = [C.POINTER(GatedRecurrenceDesc), vp]
+    L.ntk_gated_recurrence_scratch.argtypes = [i, i, i, i]
+    L.ntk_gated_recurrence_scratch.restype = C.c_size_t
     L.ntk_glu_cubic.argtypes = [vp, vp, i, i, i, f, f, f, f, vp]
     L._layers_bound = True
     return L
@@ -491,9 +493,10 @@ def gated_seam(x, y=None, g=None, yb=None, gb=None, hist=None, coef=None, norm=N
 
 
 def gated_recurrence(q, k, v, wz, H: int, dn: int, dv: int, pos0: int, decay_form: int = DECAY_GIVEN, decay_param: float = 1.0, wb=None, az=None, ab=None,
-                     unit_eps: float = 1e-6, q_scale: float = 1.0, state: Optional[np.ndarray] = None):
+                     unit_eps: float = 1e-6, q_scale: float = 1.0, state: Optional[np.ndarray] = None, prepass: bool = True):
     """-> (out [T, H * dv], state [H, dn, dv]); az: the removal rate's raw projection (None: no removal term); state: what an earlier portion left (ignored when
-    pos0 == 0; by default full of NaN so that a read at the start would show)"""
+    pos0 == 0; by default full of NaN so that a read at the start would show); prepass: give the scratch that lets longer portions form their per-token vectors
+    in a launch of their own"""
     L = _bind()
     T = q.shape[0]
     qb, kb, vb, zb = _f(q), _f(k), _f(v), _f(wz)
@@ -502,7 +505,11 @@ def gated_recurrence(q, k, v, wz, H: int, dn: int, dv: int, pos0: int, decay_for
     out = DeviceBuffer.zeros(T * H * dv * 4)
     d = GatedRecurrenceDesc(out.ptr, H * dv, qb.ptr, q.shape[1], kb.ptr, k.shape[1], vb.ptr, v.shape[1], zb.ptr, wz.shape[1], wbb.ptr if wbb else None, decay_form,
                             decay_param, azb.ptr if azb else None, az.shape[1] if az is not None else 0, abb.ptr if abb else None, unit_eps, sb.ptr, H, dn, dv, q_scale,
-                            pos0, T)
+                            pos0, T, None)
+    ns = int(L.ntk_gated_recurrence_scratch(T, H, dn, int(az is not None))) if prepass else 0
+    scr = DeviceBuffer.from_numpy(np.full(ns, np.nan, np.float32)) if ns else None
+    if scr:
+        d.scratch = scr.ptr
     check(L.ntk_gated_recurrence(C.byref(d), None), "ntk_gated_recurrence")
     return out.numpy(np.float32, T * H * dv).reshape(T, H * dv), sb.numpy(np.float32, H * dn * dv).reshape(H, dn, dv)
 

@@ -249,6 +249,8 @@ def test_decay_recurrence_whole_in_portions_and_token_by_token(H, dn, dv, delta)
     ref = ref.reshape(T, H * dv)
     out, st = Lr.gated_recurrence(q, k, v, wz, H, dn, dv, 0, **kw)          # (the state buffer starts full of NaN: position 0 must not read it)
     assert rel(out, ref) < 2e-6 and rel(st, S) < 2e-6
+    out2, st2 = Lr.gated_recurrence(q, k, v, wz, H, dn, dv, 0, prepass=False, **kw)   # the per-token vectors formed inside the walk instead of ahead of it
+    assert np.abs(out2 - out).max() <= 1e-6 * np.abs(ref).max() and rel(st2, S) < 2e-6
     for cuts in ([1] * T, [2, 9, 3, 8, 17, 1, 5], [16, 16, 13], [44, 1]):
         parts, at, st = [], 0, None
         for n in cuts:
