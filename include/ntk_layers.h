@@ -212,7 +212,8 @@ int ntk_lightning_attention(float* out, int ldo, const float* q, int ldq, const 
  *     NTK_DECAY_GIVEN          w = z
  * az (may be NULL: no removal term -- gated linear attention): a = sigmoid(az + ab), [T][H][dn] (+ ab [H*dn], may be NULL).
  * state [H][dn][dv]: read unless pos0 == 0 (a sequence starts from zeros), written at the end.  out [T][H][dv].  dn <= 1024.
- * A lane owns a few state rows of one column; tokens are walked in order, so a portion cut anywhere gives the same sums in the same order. */
+ * A lane owns a few state rows of one column and walks its tokens in order.  Without scratch a portion cut anywhere gives the same sums in the same order;
+ * with it, where a long portion's segments end changes rounding only. */
 #define NTK_DECAY_GIVEN 0
 #define NTK_DECAY_SIGMOID_ROOT 1
 #define NTK_DECAY_EXP_SIGMOID 2
@@ -227,10 +228,11 @@ typedef struct ntk_gated_recurrence_desc {
     int H, dn, dv;
     float q_scale;
     int pos0, T;
-    float* scratch;   /* F32 [>= ntk_gated_recurrence_scratch(T, H, dn, az != NULL)]: portions of more than a few tokens form their per-token vectors in a launch
-                         of their own, once per head instead of once per workgroup; NULL: always inside the walk */
+    float* scratch;   /* F32 [>= ntk_gated_recurrence_scratch(T, H, dn, dv, az != NULL)]: portions of more than a few tokens form their per-token vectors in a launch
+                         of their own, once per head instead of once per workgroup, and long portions are walked in segments side by side (their states and
+                         what the outputs are still owed are settled by two more launches); NULL: always inside the walk, tokens strictly in turn */
 } ntk_gated_recurrence_desc;
-size_t ntk_gated_recurrence_scratch(int T, int H, int dn, int removal);
+size_t ntk_gated_recurrence_scratch(int T, int H, int dn, int dv, int removal);
 int ntk_gated_recurrence(const ntk_gated_recurrence_desc* d, void* stream);
 
 /* ---- moe.hip ---------------------------------------------------------------------------------------------------------------------- */

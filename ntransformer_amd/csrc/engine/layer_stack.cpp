@@ -693,13 +693,13 @@ int LayerStackModel::alloc_buffers() {
             max_in_ = std::max<int>(max_in_, (int)m.in.out_f);
             max_hdv_ = std::max(max_hdv_, m.heads * m.vdim);
             max_rec_ = std::max(max_rec_, m.heads * m.dim);
-            rsc = std::max(rsc, ntk_gated_recurrence_scratch(chunk_, m.heads, m.dim, 0));
+            rsc = std::max(rsc, ntk_gated_recurrence_scratch(chunk_, m.heads, m.dim, m.vdim, 0));
         } else {
             const ParallelMixer& m = L.par;
             max_in_ = std::max<int>(max_in_, (int)m.in.out_f);
             max_hdv_ = std::max<int>(max_hdv_, (int)m.o.in_f);
             max_rec_ = std::max(max_rec_, m.right.heads * m.right.dim);
-            rsc = std::max(rsc, ntk_gated_recurrence_scratch(chunk_, m.right.heads, m.right.dim, 1));
+            rsc = std::max(rsc, ntk_gated_recurrence_scratch(chunk_, m.right.heads, m.right.dim, m.right.dim, 1));
             wsc = std::max(wsc, ntk_window_attention_scratch(chunk_, m.left.heads, 1, m.left.vdim, opt_.max_context));
         }
         if (form_.gated && L.has_mlp) max_gu2_ = std::max<int>(max_gu2_, (int)L.gff.in.out_f), max_ffn_ = std::max(max_ffn_, L.gff.ff);

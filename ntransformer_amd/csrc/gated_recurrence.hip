@@ -13,7 +13,12 @@
 // requested into registers before the current batch is walked, so their latency hides behind the walk.
 // Portions of more than a few tokens run a pre-pass first (one wave per token and head, the whole chip at once) that leaves those vectors ready-made in a
 // packed buffer [T][H][vectors][dn]: the walk's staging is then a copy, and what a head's workgroups would each have recomputed is computed once.
-// The walk is the same whatever the portion: a sequence cut anywhere gives the same sums in the same order.
+// Long portions are walked in SEGMENTS side by side (the chain from token to token is latency, and a wave that waits costs its neighbours nothing): every
+// segment but the first starts from a zero state, and dn extra columns that start as the identity and take no k v^T ride along -- they hold P, the product
+// of the segment's transitions M_t = diag(w_t) - (a_t u_t) u_t^T, and their outputs are P_t^T q_t.  Then x(g + 1) = P(g) x(g) + L(g) hands the true state
+// from segment to segment (recurrence_chain_kernel, a few small products in turn) and out_t += x(g)^T (P_t^T q_t) settles what every token's output was
+// still owed (recurrence_owed_kernel).  Only products of decays <= 1 appear, nothing is divided by a decay: no overflow whatever the decays are.
+// Within a segment the walk is the same whatever the portion; where the segments' borders fall changes the order of the sums, i.e. rounding only.
 #include <algorithm>
 #include "common.hip.h"
 #include "../../include/ntk_layers.h"
@@ -32,6 +37,12 @@ struct RecArgs {
     float q_scale;
     int pos0, T, TB;
     float* packed;                   // [T][H][NV][dn] ready-made vectors (q * scale, k, w (, u, a * u)), or NULL: formed while staging
+    // segments walked side by side (nseg > 1, packed only): segment g owns tokens [g * seg_len, (g + 1) * seg_len)
+    int nseg, seg_len;
+    float* rbuf;                     // [T][H][dn]: P_t^T q_t, P_t the product of the segment's transitions up to t
+    float* pbuf;                     // [nseg][H][dn][dn]: the segment's whole transition
+    float* lbuf;                     // [nseg][H][dn][dv]: the state the segment's own tokens leave (segment 0: from the sequence's state)
+    float* sbuf;                     // [nseg][H][dn][dv]: the state at the segment's start
 };
 
 constexpr int kRecFewTokens = 8;  // up to this many tokens (decoding) the walk forms its vectors itself: one launch
@@ -94,14 +105,19 @@ __global__ __launch_bounds__(64 * NW) void gated_recurrence_kernel(const RecArgs
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int cl = lane / SPLIT, rg = lane % SPLIT;
     const int h = blockIdx.y, c0 = blockIdx.x * CB, c = c0 + wave * CW + cl;
-    const bool col_ok = c < a.dv;
+    // a segment of the portion; with several segments dn more columns ride along that start as the identity and receive no k v^T: they hold the product
+    // of the segment's transitions, and their outputs are what the state at the segment's start still owes every token's output
+    const int sg = blockIdx.z, tbase = sg * a.seg_len, T = min(a.T - tbase, a.seg_len);
+    const int ncols = (DELTA && a.nseg > 1) ? a.dv + a.dn : a.dv;
+    const bool col_ok = c < ncols, aug = c >= a.dv;
     // ---- the state slice: rows rg * RP + i of column c
     float S[RP];
     float* st = a.state + ((long long)h * a.dn) * a.dv + c;
 #pragma unroll
     for (int i = 0; i < RP; ++i) {
         const int r = rg * RP + i;
-        S[i] = (a.pos0 > 0 && col_ok && r < a.dn) ? st[(long long)r * a.dv] : 0.0f;
+        if (aug) S[i] = r == c - a.dv ? 1.0f : 0.0f;
+        else S[i] = (sg == 0 && a.pos0 > 0 && col_ok && r < a.dn) ? st[(long long)r * a.dv] : 0.0f;
     }
     // ---- the two slots behind a full batch: a token that leaves the state as it is and asks for nothing
     for (int e = threadIdx.x; e < EXTRA * NV * DL; e += NT) Vec[(size_t)a.TB * NV * DL + e] = (e % (NV * DL)) / DL == 2 ? 1.0f : 0.0f;
@@ -113,7 +129,7 @@ __global__ __launch_bounds__(64 * NW) void gated_recurrence_kernel(const RecArgs
         for (int u = 0; u < REC_PF; ++u) {
             const int idx = threadIdx.x + NT * u, tb = idx / DP, d = idx % DP;
             const bool ok = tb < nb && d < a.dn;
-            const long long t = t0 + tb;
+            const long long t = tbase + t0 + tb;
             if constexpr (PACKED) {
                 const float* src = a.packed + ((t * a.H + h) * NV) * a.dn + d;
                 pq[u] = ok ? src[0] : 0.0f;
@@ -130,7 +146,7 @@ __global__ __launch_bounds__(64 * NW) void gated_recurrence_kernel(const RecArgs
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const int idx = threadIdx.x + NT * u, tb = idx / CB, cc = idx % CB;
-            pv[u] = (tb < nb && c0 + cc < a.dv) ? a.v[(long long)(t0 + tb) * a.ldv + (long long)h * a.dv + c0 + cc] : 0.0f;
+            pv[u] = (tb < nb && c0 + cc < a.dv) ? a.v[(long long)(tbase + t0 + tb) * a.ldv + (long long)h * a.dv + c0 + cc] : 0.0f;
         }
     };
     auto stage = [&](int nb) {
@@ -171,13 +187,13 @@ __global__ __launch_bounds__(64 * NW) void gated_recurrence_kernel(const RecArgs
             }
         }
     };
-    request(0, min(a.TB, a.T));
-    for (int t0 = 0; t0 < a.T; t0 += a.TB) {
-        const int nb = min(a.TB, a.T - t0);
+    request(0, min(a.TB, T));
+    for (int t0 = 0; t0 < T; t0 += a.TB) {
+        const int nb = min(a.TB, T - t0);
         __syncthreads();                                 // the previous batch has been walked by every wave
         stage(nb);
         __syncthreads();
-        if (t0 + a.TB < a.T) request(t0 + a.TB, min(a.TB, a.T - t0 - a.TB));
+        if (t0 + a.TB < T) request(t0 + a.TB, min(a.TB, T - t0 - a.TB));
         // The walk.  A token's vectors leave LDS one token AHEAD of their use (a second register set while the rows per lane are few), so the only chain from
         // token to token is the state's own: u^T S, its reduction, the update.
         auto load_tok = [&](int tb, TokVec<RP, DELTA>& x) {
@@ -214,7 +230,8 @@ __global__ __launch_bounds__(64 * NW) void gated_recurrence_kernel(const RecArgs
             for (int i = 0; i < RP; i += 2) { o0 = fmaf(S[i], x.q[i], o0); o1 = fmaf(S[i + 1], x.q[i + 1], o1); }
             return o0 + o1;
         };
-        float* orow = a.out + (long long)t0 * a.ldo + (long long)h * a.dv + c;
+        const long long ostep = aug ? (long long)a.H * a.dn : a.ldo;
+        float* orow = aug ? a.rbuf + (long long)(tbase + t0) * ostep + (long long)h * a.dn + (c - a.dv) : a.out + (long long)(tbase + t0) * ostep + (long long)h * a.dv + c;
         if constexpr (RP <= 8) {
             // two tokens per pass of the loop, no branch inside: the slots behind a batch's last token hold a token that changes nothing (decay one, the rest zero),
             // so both register sets are always loaded and walked, and only the stores look at the token's number
@@ -227,8 +244,8 @@ __global__ __launch_bounds__(64 * NW) void gated_recurrence_kernel(const RecArgs
                 const float ob = step(x1);
                 const float ra = group_sum<SPLIT>(oa), rb = group_sum<SPLIT>(ob);
                 if (rg == 0 && col_ok) {
-                    orow[(long long)tb * a.ldo] = ra;
-                    if (tb + 1 < nb) orow[(long long)(tb + 1) * a.ldo] = rb;
+                    orow[tb * ostep] = ra;
+                    if (tb + 1 < nb) orow[(tb + 1) * ostep] = rb;
                 }
             }
         } else {
@@ -236,14 +253,136 @@ __global__ __launch_bounds__(64 * NW) void gated_recurrence_kernel(const RecArgs
                 TokVec<RP, DELTA> cur;
                 load_tok(tb, cur);
                 const float o = group_sum<SPLIT>(step(cur));
-                if (rg == 0 && col_ok) orow[(long long)tb * a.ldo] = o;
+                if (rg == 0 && col_ok) orow[tb * ostep] = o;
             }
         }
+    }
+    // ---- what the walk leaves: the sequence's state, or with several segments the segment's own end state and its whole transition
+    float* end = st;
+    long long estep = a.dv;
+    if (a.nseg > 1) {
+        if (aug) { end = a.pbuf + (((long long)sg * a.H + h) * a.dn) * a.dn + (c - a.dv); estep = a.dn; }
+        else end = a.lbuf + (((long long)sg * a.H + h) * a.dn) * a.dv + c;
     }
 #pragma unroll
     for (int i = 0; i < RP; ++i) {
         const int r = rg * RP + i;
-        if (col_ok && r < a.dn) st[(long long)r * a.dv] = S[i];
+        if (col_ok && r < a.dn) end[r * estep] = S[i];
+    }
+}
+
+// Without the removal term a segment's transition is diagonal: P_t = diag(B_t), B_t the running product of the segment's decays per channel.  A thread
+// per (segment, head, channel) walks its tokens (eight tokens' loads in flight at a time): r_t = q_t * B_t, and the segment's whole product at the end.
+__global__ __launch_bounds__(64) void recurrence_cumdecay_kernel(const RecArgs a) {
+    const int d = blockIdx.x * 64 + threadIdx.x, h = blockIdx.y, g = blockIdx.z;
+    if (d >= a.dn) return;
+    const int t0 = g * a.seg_len, t1 = min(a.T, t0 + a.seg_len);
+    float B = 1.0f;
+    for (int t = t0; t < t1; t += 8) {
+        float w[8], q[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float* src = a.packed + (((long long)min(t + j, t1 - 1) * a.H + h) * 3) * a.dn + d;
+            q[j] = src[0];
+            w[j] = src[2 * a.dn];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            if (t + j < t1) { B *= w[j]; a.rbuf[((long long)(t + j) * a.H + h) * a.dn + d] = q[j] * B; }
+    }
+    a.pbuf[((long long)g * a.H + h) * a.dn + d] = B;
+}
+
+// The states at the segments' starts, one after the other: x(1) = what segment 0 left (it started from the sequence's state), x(g + 1) = P(g) x(g) + L(g).
+// A workgroup owns 16 columns of one head: lane = (column, one of 4 row groups), wave = 4 more row groups, a thread the rows of its group (every 16th);
+// x and the segment's P in LDS.  DIAG: P is a vector (no removal term).
+template <bool DIAG>
+__global__ __launch_bounds__(256) void recurrence_chain_kernel(const RecArgs a) {
+    extern __shared__ __attribute__((aligned(16))) float cl_[];
+    const int DS = ((a.dn + 3) & ~3) + 4;                // floats per row of P in LDS
+    float* x0 = cl_;                                     // [dn][16]
+    float* x1 = x0 + a.dn * 16;
+    float* Pl = x1 + a.dn * 16;                          // [dn][DS]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = blockIdx.y;
+    const int cc = lane & 15, rgrp = wave * 4 + (lane >> 4), c = blockIdx.x * 16 + cc;
+    const bool ok = c < a.dv;
+    const long long hs = (long long)a.dn * a.dv;
+    for (int r = rgrp; r < a.dn; r += 16) x0[r * 16 + cc] = ok ? a.lbuf[(long long)h * hs + (long long)r * a.dv + c] : 0.0f;
+    for (int g = 1; g < a.nseg; ++g) {
+        const float* L = a.lbuf + ((long long)g * a.H + h) * hs;
+        float* Sg = a.sbuf + ((long long)g * a.H + h) * hs;
+        if constexpr (DIAG) {
+            const float* Pd = a.pbuf + ((long long)g * a.H + h) * a.dn;
+            for (int r = rgrp; r < a.dn; r += 16) {      // (a thread's own entries only: no barrier between the segments)
+                const float cur = x0[r * 16 + cc];
+                if (ok) Sg[(long long)r * a.dv + c] = cur;
+                x0[r * 16 + cc] = fmaf(Pd[r], cur, ok ? L[(long long)r * a.dv + c] : 0.0f);
+            }
+        } else {
+            const float* P = a.pbuf + ((long long)g * a.H + h) * a.dn * a.dn;
+            __syncthreads();                             // the previous segment's readers of Pl and x1 are done
+            for (int e = threadIdx.x; e < a.dn * a.dn; e += 256) Pl[(e / a.dn) * DS + e % a.dn] = P[e];
+            if (DS - 4 > a.dn)
+                for (int r = threadIdx.x; r < a.dn; r += 256)
+                    for (int k = a.dn; k < DS - 4; ++k) Pl[r * DS + k] = 0.0f;
+            __syncthreads();
+            float acc[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
+            for (int k = 0; k < a.dn; k += 4) {          // (entries of P past dn are zero, x is read below dn only)
+                const float xa = x0[k * 16 + cc], xb = k + 1 < a.dn ? x0[(k + 1) * 16 + cc] : 0.0f, xc = k + 2 < a.dn ? x0[(k + 2) * 16 + cc] : 0.0f,
+                            xd = k + 3 < a.dn ? x0[(k + 3) * 16 + cc] : 0.0f;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int r = rgrp + 16 * j;
+                    if (r < a.dn) {
+                        const float4 p4 = *reinterpret_cast<const float4*>(Pl + r * DS + k);
+                        acc[j] = fmaf(p4.x, xa, acc[j]); acc[j] = fmaf(p4.y, xb, acc[j]); acc[j] = fmaf(p4.z, xc, acc[j]); acc[j] = fmaf(p4.w, xd, acc[j]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int r = rgrp + 16 * j;
+                if (r < a.dn) {
+                    if (ok) Sg[(long long)r * a.dv + c] = x0[r * 16 + cc];
+                    x1[r * 16 + cc] = acc[j] + (ok ? L[(long long)r * a.dv + c] : 0.0f);
+                }
+            }
+            float* t = x0; x0 = x1; x1 = t;
+        }
+    }
+    if constexpr (!DIAG) __syncthreads();
+    for (int r = rgrp; r < a.dn; r += 16)
+        if (ok) a.state[(long long)h * hs + (long long)r * a.dv + c] = x0[r * 16 + cc];
+}
+
+// out[t] += S(g)^T r[t] for the tokens of segments g >= 1: a workgroup owns 16 tokens of one head (r rows in LDS), lane = column, wave = 4 tokens
+__global__ __launch_bounds__(256) void recurrence_owed_kernel(const RecArgs a) {
+    extern __shared__ float rs[];                        // [16][dn]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = blockIdx.y;
+    const int g = 1 + blockIdx.x / ((a.seg_len + 15) / 16), tile = blockIdx.x % ((a.seg_len + 15) / 16);
+    const int t0 = g * a.seg_len + tile * 16, tend = min(a.T, (g + 1) * a.seg_len);
+    if (t0 >= tend) return;                              // (uniform over the workgroup)
+    for (int e = threadIdx.x; e < 16 * a.dn; e += 256) {
+        const int t = t0 + e / a.dn;
+        rs[e] = t < tend ? a.rbuf[((long long)t * a.H + h) * a.dn + e % a.dn] : 0.0f;
+    }
+    __syncthreads();
+    const float* Sg = a.sbuf + ((long long)g * a.H + h) * a.dn * a.dv;
+    const float* r4 = rs + wave * 4 * a.dn;
+    for (int c = lane; c < a.dv; c += 64) {
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int k = 0; k < a.dn; ++k) {
+            const float sv = Sg[(long long)k * a.dv + c];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] = fmaf(r4[j * a.dn + k], sv, acc[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int t = t0 + wave * 4 + j;
+            if (t < tend) a.out[(long long)t * a.ldo + (long long)h * a.dv + c] += acc[j];
+        }
     }
 }
 
@@ -260,7 +399,8 @@ static int launch_rec_waves(const RecArgs& a0, hipStream_t s) {
     tb = std::min(tb, std::max(a.T, 1));
     a.TB = std::max(tb, 1);
     const size_t lds = (size_t)(a.TB + extra) * (NV * DL + CB) * sizeof(float);
-    const dim3 grid((a.dv + CB - 1) / CB, a.H);
+    const int ncols = (delta && a.nseg > 1) ? a.dv + a.dn : a.dv;
+    const dim3 grid((ncols + CB - 1) / CB, a.H, a.nseg);
     if (a.packed) {
         if (delta) hipLaunchKernelGGL(gated_recurrence_prepare_kernel<true>, dim3(a.T * a.H), dim3(64), 0, s, a);
         else hipLaunchKernelGGL(gated_recurrence_prepare_kernel<false>, dim3(a.T * a.H), dim3(64), 0, s, a);
@@ -268,6 +408,22 @@ static int launch_rec_waves(const RecArgs& a0, hipStream_t s) {
         if (st != NTK_OK) return st;
         if (delta) hipLaunchKernelGGL((gated_recurrence_kernel<SPLIT, RP, true, true, NW>), grid, dim3(NT), lds, s, a);
         else hipLaunchKernelGGL((gated_recurrence_kernel<SPLIT, RP, false, true, NW>), grid, dim3(NT), lds, s, a);
+        if (a.nseg == 1) return last_launch_status();
+        const dim3 cgrid((a.dv + 15) / 16, a.H);
+        if (delta) {
+            const size_t clds = ((size_t)2 * a.dn * 16 + (size_t)a.dn * (((a.dn + 3) & ~3) + 4)) * sizeof(float);
+            static bool raised = false;   // (idempotent: a race sets the same attribute twice)
+            if (!raised) {
+                NTK_HIP_TRY(hipFuncSetAttribute((const void*)recurrence_chain_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+                raised = true;
+            }
+            hipLaunchKernelGGL(recurrence_chain_kernel<false>, cgrid, dim3(256), clds, s, a);
+        } else {
+            hipLaunchKernelGGL(recurrence_cumdecay_kernel, dim3((a.dn + 63) / 64, a.H, a.nseg), dim3(64), 0, s, a);
+            hipLaunchKernelGGL(recurrence_chain_kernel<true>, cgrid, dim3(256), (size_t)2 * a.dn * 16 * sizeof(float), s, a);
+        }
+        const int tiles = (a.seg_len + 15) / 16;
+        hipLaunchKernelGGL(recurrence_owed_kernel, dim3((a.nseg - 1) * tiles, a.H), dim3(256), (size_t)16 * a.dn * sizeof(float), s, a);
         return last_launch_status();
     }
     if (delta) hipLaunchKernelGGL((gated_recurrence_kernel<SPLIT, RP, true, false, NW>), grid, dim3(NT), lds, s, a);
@@ -279,7 +435,7 @@ static int launch_rec_waves(const RecArgs& a0, hipStream_t s) {
 // that the walk -- one chain per column, nothing to gain from a second wave on the same column -- spreads over the chip
 template <int SPLIT, int RP>
 static int launch_rec(const RecArgs& a, hipStream_t s) {
-    const long long col_groups = (long long)a.H * ((a.dv + 64 / SPLIT - 1) / (64 / SPLIT));   // waves of the launch
+    const long long col_groups = (long long)a.H * ((((a.az && a.nseg > 1) ? a.dv + a.dn : a.dv) + 64 / SPLIT - 1) / (64 / SPLIT)) * a.nseg;   // waves of the launch
     if (col_groups >= 4 * 256) return launch_rec_waves<SPLIT, RP, 4>(a, s);
     if (col_groups >= 2 * 256) return launch_rec_waves<SPLIT, RP, 2>(a, s);
     return launch_rec_waves<SPLIT, RP, 1>(a, s);
@@ -289,8 +445,24 @@ static int launch_rec(const RecArgs& a, hipStream_t s) {
 
 using namespace ntk;
 
-size_t ntk_gated_recurrence_scratch(int T, int H, int dn, int removal) {
-    return T > kRecFewTokens ? (size_t)T * H * (removal ? 5 : 3) * dn : 0;
+// segments of a portion: at least kRecSegTokens tokens each, at most kRecMaxSegs; channels beyond 128 stay in one segment (the transition of a segment
+// is a dn x dn matrix per head)
+// ... and no more segments than fill the chip a few waves deep: beyond that the walk is bound by what it issues, not by its chain, and the extra columns
+// and the settling launches only cost
+constexpr int kRecSegTokens = 64, kRecMaxSegs = 16, kRecWaves = 4096;
+static int rec_segments(int T, int H, int dn, int dv, bool removal) {
+    if (dn > 128 || dv > 1024) return 1;
+    const long long waves = ((long long)H * (dv + (removal ? dn : 0)) + 3) / 4;        // of one segment, 16 lanes per column
+    const int by_chip = (int)std::max<long long>(1, kRecWaves / std::max<long long>(waves, 1));
+    return std::max(1, std::min(std::min(kRecMaxSegs, by_chip), T / kRecSegTokens));
+}
+
+size_t ntk_gated_recurrence_scratch(int T, int H, int dn, int dv, int removal) {
+    if (T <= kRecFewTokens) return 0;
+    size_t n = (size_t)T * H * (removal ? 5 : 3) * dn;
+    const int ns = rec_segments(T, H, dn, dv, removal != 0);
+    if (ns > 1) n += (size_t)T * H * dn + (size_t)ns * H * dn * dn + 2 * (size_t)ns * H * dn * dv;
+    return n;
 }
 
 int ntk_gated_recurrence(const ntk_gated_recurrence_desc* d, void* stream) {
@@ -302,7 +474,18 @@ int ntk_gated_recurrence(const ntk_gated_recurrence_desc* d, void* stream) {
     if (d->ldq < hd || d->ldk < hd || d->ldw < hd || (d->az && d->lda < hd) || d->ldv < d->H * d->dv || d->ldo < d->H * d->dv) return NTK_E_SHAPE;
     if (d->T == 0) return NTK_OK;
     RecArgs a{d->out, d->ldo, d->q, d->ldq, d->k, d->ldk, d->v, d->ldv, d->wz, d->ldw, d->wb, d->decay_form, d->decay_param, d->az, d->lda, d->ab, d->unit_eps,
-              d->state, d->H, d->dn, d->dv, d->q_scale, d->pos0, d->T, 0, d->T > kRecFewTokens ? d->scratch : nullptr};
+              d->state, d->H, d->dn, d->dv, d->q_scale, d->pos0, d->T, 0, d->T > kRecFewTokens ? d->scratch : nullptr, 1, d->T, nullptr, nullptr, nullptr, nullptr};
+    if (a.packed) {
+        a.nseg = rec_segments(d->T, d->H, d->dn, d->dv, d->az != nullptr);
+        if (a.nseg > 1) {
+            a.seg_len = (d->T + a.nseg - 1) / a.nseg;
+            a.nseg = (d->T + a.seg_len - 1) / a.seg_len;
+            a.rbuf = a.packed + (size_t)d->T * d->H * (d->az ? 5 : 3) * d->dn;
+            a.pbuf = a.rbuf + (size_t)d->T * d->H * d->dn;
+            a.lbuf = a.pbuf + (size_t)a.nseg * d->H * d->dn * d->dn;
+            a.sbuf = a.lbuf + (size_t)a.nseg * d->H * d->dn * d->dv;
+        }
+    }
     hipStream_t s = resolve_stream(stream);
     // 16 lanes share a column (their sums meet in DPP steps inside a 16-lane row, no trip through LDS on the chain from token to token); rows per lane: the
     // smallest of 4 / 8 / 16 / 32 that covers the head's channels; beyond 512 channels 32 lanes per column.

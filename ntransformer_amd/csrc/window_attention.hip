@@ -1,5 +1,6 @@
 // window_attention.hip -- grouped-query softmax attention over a cache of rotated keys and values: causal, optional sliding window, one or two score
-// maps per head over the same values (two maps: the differential pair out = a_0 - lambda * a_1), optional unit norm of every head's output.
+// maps per head over the same values (two maps: the differential pair out = a_0 - lambda * a_1), optional unit norm of every head's output, optional
+// learned bias by bucketed distance on the scaled score (a table of distances -> buckets, a table of buckets x heads).
 //
 // Cache row of a position: [G][maps][dn] rotated keys | [G][dv] values, F32.  Scores, softmax, weights and sums are F32 on the vector units.
 // A workgroup owns 16 (token, head) rows of ONE key/value head -- consecutive tokens times the heads that share it, so a key or value slab that was

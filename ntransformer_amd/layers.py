@@ -102,7 +102,7 @@ def _bind():
     L.ntk_gated_seam.argtypes = [C.POINTER(GatedSeamDesc), vp]
     L.ntk_window_prepare_biased.argtypes = [vp, i, vp, i, vp, i, vp, i, i, i, i, i, i, C.POINTER(Rotary), vp, vp, vp, f, C.c_double, i, i, vp]
     L.ntk_gated_recurrence.argtypes = [C.POINTER(GatedRecurrenceDesc), vp]
-    L.ntk_gated_recurrence_scratch.argtypes = [i, i, i, i]
+    L.ntk_gated_recurrence_scratch.argtypes = [i, i, i, i, i]
     L.ntk_gated_recurrence_scratch.restype = C.c_size_t
     L.ntk_glu_cubic.argtypes = [vp, vp, i, i, i, f, f, f, f, vp]
     L._layers_bound = True
@@ -506,7 +506,7 @@ def gated_recurrence(q, k, v, wz, H: int, dn: int, dv: int, pos0: int, decay_for
     d = GatedRecurrenceDesc(out.ptr, H * dv, qb.ptr, q.shape[1], kb.ptr, k.shape[1], vb.ptr, v.shape[1], zb.ptr, wz.shape[1], wbb.ptr if wbb else None, decay_form,
                             decay_param, azb.ptr if azb else None, az.shape[1] if az is not None else 0, abb.ptr if abb else None, unit_eps, sb.ptr, H, dn, dv, q_scale,
                             pos0, T, None)
-    ns = int(L.ntk_gated_recurrence_scratch(T, H, dn, int(az is not None))) if prepass else 0
+    ns = int(L.ntk_gated_recurrence_scratch(T, H, dn, dv, int(az is not None))) if prepass else 0
     scr = DeviceBuffer.from_numpy(np.full(ns, np.nan, np.float32)) if ns else None
     if scr:
         d.scratch = scr.ptr

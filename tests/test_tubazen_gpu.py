@@ -262,6 +262,38 @@ def test_decay_recurrence_whole_in_portions_and_token_by_token(H, dn, dv, delta)
         assert np.abs(np.concatenate(parts) - out).max() <= 1e-6 * np.abs(ref).max()      # the same sums in the same order, whatever the cut
 
 
+@pytest.mark.parametrize("H,dn,dv", [(2, 9, 11), (3, 64, 64), (1, 128, 70), (2, 96, 128), (1, 130, 20)])
+@pytest.mark.parametrize("delta", [False, True])
+def test_long_portions_walk_in_segments_side_by_side(H, dn, dv, delta):
+    """portions long enough to be cut into segments that start from nothing and are settled afterwards (the state handed from segment to segment, every
+    output given what the state at its segment's start still owed it) against the walk in turn and the oracle; from a sequence's start and from a state;
+    lengths that leave a short last segment; heads too wide for segments stay in turn"""
+    from ntransformer_amd import layers as Lr
+    g = np.random.default_rng(H * dn + dv + delta)
+    T0, T = 37, 333
+    q, k, v, wz, az, wb, ab = _recurrence_inputs(g, T0 + T, H, dn, dv, 2.0)
+    z = (wz + wb).astype(np.float64).reshape(-1, H, dn)
+    if delta:
+        kw = dict(decay_form=Lr.DECAY_EXP_SIGMOID, decay_param=0.6, wb=wb, ab=ab, unit_eps=1e-6)
+        decay, removal = np.exp(-0.6 * O.sigmoid(z)), O.sigmoid((az + ab).astype(np.float64)).reshape(-1, H, dn)
+    else:
+        kw = dict(decay_form=Lr.DECAY_SIGMOID_ROOT, decay_param=8.0, wb=wb)
+        decay, removal = O.sigmoid(z) ** (1 / 8.0), None
+    ref, S = O.decay_recurrence(q.astype(np.float64).reshape(-1, H, dn), k.astype(np.float64).reshape(-1, H, dn), v.astype(np.float64).reshape(-1, H, dv), decay, removal, 1e-6)
+    ref = ref.reshape(-1, H * dv)
+    run = lambda a, b, st, **more: Lr.gated_recurrence(q[a:b], k[a:b], v[a:b], wz[a:b], H, dn, dv, a, state=st, az=az[a:b] if delta else None, **dict(kw, **more))
+    whole, st = run(0, T0 + T, None)
+    assert rel(whole, ref) < 3e-6 and rel(st, S) < 3e-6
+    turn, st2 = run(0, T0 + T, None, prepass=False)
+    assert rel(whole, turn) < 3e-6 and rel(st, st2) < 3e-6
+    head, st = run(0, T0, None)
+    tail, st = run(T0, T0 + T, st)                                          # the first segment starts from the sequence's state
+    assert rel(np.concatenate([head, tail]), ref) < 3e-6 and rel(st, S) < 3e-6
+    for n in (128, 129, 191):                                               # two segments of 64, of 65, of 96 and 95
+        part, _ = run(0, n, None)
+        assert rel(part, ref[:n]) < 3e-6, n
+
+
 def test_decay_forms_at_their_ends_and_a_given_decay():
     from ntransformer_amd import layers as Lr
     T, H, dn, dv = 6, 1, 4, 3
