@@ -272,22 +272,22 @@ __global__ __launch_bounds__(64 * NW) void gated_recurrence_kernel(const RecArgs
 }
 
 // Without the removal term a segment's transition is diagonal: P_t = diag(B_t), B_t the running product of the segment's decays per channel.  A thread
-// per (segment, head, channel) walks its tokens (eight tokens' loads in flight at a time): r_t = q_t * B_t, and the segment's whole product at the end.
+// per (segment, head, channel) walks its tokens (sixteen tokens' loads in flight at a time): r_t = q_t * B_t, and the segment's whole product at the end.
 __global__ __launch_bounds__(64) void recurrence_cumdecay_kernel(const RecArgs a) {
     const int d = blockIdx.x * 64 + threadIdx.x, h = blockIdx.y, g = blockIdx.z;
     if (d >= a.dn) return;
     const int t0 = g * a.seg_len, t1 = min(a.T, t0 + a.seg_len);
     float B = 1.0f;
-    for (int t = t0; t < t1; t += 8) {
-        float w[8], q[8];
+    for (int t = t0; t < t1; t += 16) {
+        float w[16], q[16];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < 16; ++j) {
             const float* src = a.packed + (((long long)min(t + j, t1 - 1) * a.H + h) * 3) * a.dn + d;
             q[j] = src[0];
             w[j] = src[2 * a.dn];
         }
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
+        for (int j = 0; j < 16; ++j)
             if (t + j < t1) { B *= w[j]; a.rbuf[((long long)(t + j) * a.H + h) * a.dn + d] = q[j] * B; }
     }
     a.pbuf[((long long)g * a.H + h) * a.dn + d] = B;
@@ -449,7 +449,7 @@ using namespace ntk;
 // is a dn x dn matrix per head)
 // ... and no more segments than fill the chip a few waves deep: beyond that the walk is bound by what it issues, not by its chain, and the extra columns
 // and the settling launches only cost
-constexpr int kRecSegTokens = 64, kRecMaxSegs = 16, kRecWaves = 4096;
+constexpr int kRecSegTokens = 64, kRecMaxSegs = 16, kRecWaves = 2048;
 static int rec_segments(int T, int H, int dn, int dv, bool removal) {
     if (dn > 128 || dv > 1024) return 1;
     const long long waves = ((long long)H * (dv + (removal ? dn : 0)) + 3) / 4;        // of one segment, 16 lanes per column
