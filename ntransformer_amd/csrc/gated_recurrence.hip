@@ -295,8 +295,9 @@ __global__ __launch_bounds__(64) void recurrence_cumdecay_kernel(const RecArgs a
 
 // The states at the segments' starts, one after the other: x(1) = what segment 0 left (it started from the sequence's state), x(g + 1) = P(g) x(g) + L(g).
 // A workgroup owns 16 columns of one head: lane = (column, one of 4 row groups), wave = 4 more row groups, a thread the rows of its group (every 16th);
-// x and the segment's P in LDS.  DIAG: P is a vector (no removal term).
-template <bool DIAG>
+// x and the segment's P in LDS; the NEXT segment's P and L are requested into registers (PFN floats of P per thread) while the current product runs, so a
+// step waits for its own arithmetic only.  DIAG: P is a vector (no removal term).
+template <bool DIAG, int PFN>
 __global__ __launch_bounds__(256) void recurrence_chain_kernel(const RecArgs a) {
     extern __shared__ __attribute__((aligned(16))) float cl_[];
     const int DS = ((a.dn + 3) & ~3) + 4;                // floats per row of P in LDS
@@ -308,6 +309,16 @@ __global__ __launch_bounds__(256) void recurrence_chain_kernel(const RecArgs a) 
     const bool ok = c < a.dv;
     const long long hs = (long long)a.dn * a.dv;
     for (int r = rgrp; r < a.dn; r += 16) x0[r * 16 + cc] = ok ? a.lbuf[(long long)h * hs + (long long)r * a.dv + c] : 0.0f;
+    float pn[PFN], ln[8];
+    auto request = [&](int g) {
+        const float* P = a.pbuf + ((long long)g * a.H + h) * a.dn * a.dn;
+        const float* L = a.lbuf + ((long long)g * a.H + h) * hs;
+#pragma unroll
+        for (int u = 0; u < PFN; ++u) { const int e = threadIdx.x + 256 * u; pn[u] = e < a.dn * a.dn ? P[e] : 0.0f; }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { const int r = rgrp + 16 * j; ln[j] = (ok && r < a.dn) ? L[(long long)r * a.dv + c] : 0.0f; }
+    };
+    if constexpr (!DIAG) { if (a.nseg > 1) request(1); }
     for (int g = 1; g < a.nseg; ++g) {
         const float* L = a.lbuf + ((long long)g * a.H + h) * hs;
         float* Sg = a.sbuf + ((long long)g * a.H + h) * hs;
@@ -319,9 +330,13 @@ __global__ __launch_bounds__(256) void recurrence_chain_kernel(const RecArgs a) 
                 x0[r * 16 + cc] = fmaf(Pd[r], cur, ok ? L[(long long)r * a.dv + c] : 0.0f);
             }
         } else {
-            const float* P = a.pbuf + ((long long)g * a.H + h) * a.dn * a.dn;
             __syncthreads();                             // the previous segment's readers of Pl and x1 are done
-            for (int e = threadIdx.x; e < a.dn * a.dn; e += 256) Pl[(e / a.dn) * DS + e % a.dn] = P[e];
+            float lv[8];
+#pragma unroll
+            for (int u = 0; u < PFN; ++u) { const int e = threadIdx.x + 256 * u; if (e < a.dn * a.dn) Pl[(e / a.dn) * DS + e % a.dn] = pn[u]; }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) lv[j] = ln[j];
+            if (g + 1 < a.nseg) request(g + 1);
             if (DS - 4 > a.dn)
                 for (int r = threadIdx.x; r < a.dn; r += 256)
                     for (int k = a.dn; k < DS - 4; ++k) Pl[r * DS + k] = 0.0f;
@@ -346,7 +361,7 @@ __global__ __launch_bounds__(256) void recurrence_chain_kernel(const RecArgs a) 
                 const int r = rgrp + 16 * j;
                 if (r < a.dn) {
                     if (ok) Sg[(long long)r * a.dv + c] = x0[r * 16 + cc];
-                    x1[r * 16 + cc] = acc[j] + (ok ? L[(long long)r * a.dv + c] : 0.0f);
+                    x1[r * 16 + cc] = acc[j] + lv[j];
                 }
             }
             float* t = x0; x0 = x1; x1 = t;
@@ -414,13 +429,14 @@ static int launch_rec_waves(const RecArgs& a0, hipStream_t s) {
             const size_t clds = ((size_t)2 * a.dn * 16 + (size_t)a.dn * (((a.dn + 3) & ~3) + 4)) * sizeof(float);
             static bool raised = false;   // (idempotent: a race sets the same attribute twice)
             if (!raised) {
-                NTK_HIP_TRY(hipFuncSetAttribute((const void*)recurrence_chain_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+                NTK_HIP_TRY(hipFuncSetAttribute((const void*)recurrence_chain_kernel<false, 64>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
                 raised = true;
             }
-            hipLaunchKernelGGL(recurrence_chain_kernel<false>, cgrid, dim3(256), clds, s, a);
+            if (a.dn <= 64) hipLaunchKernelGGL((recurrence_chain_kernel<false, 16>), cgrid, dim3(256), clds, s, a);
+            else hipLaunchKernelGGL((recurrence_chain_kernel<false, 64>), cgrid, dim3(256), clds, s, a);
         } else {
             hipLaunchKernelGGL(recurrence_cumdecay_kernel, dim3((a.dn + 63) / 64, a.H, a.nseg), dim3(64), 0, s, a);
-            hipLaunchKernelGGL(recurrence_chain_kernel<true>, cgrid, dim3(256), (size_t)2 * a.dn * 16 * sizeof(float), s, a);
+            hipLaunchKernelGGL((recurrence_chain_kernel<true, 1>), cgrid, dim3(256), (size_t)2 * a.dn * 16 * sizeof(float), s, a);
         }
         const int tiles = (a.seg_len + 15) / 16;
         hipLaunchKernelGGL(recurrence_owed_kernel, dim3((a.nseg - 1) * tiles, a.H), dim3(256), (size_t)16 * a.dn * sizeof(float), s, a);
