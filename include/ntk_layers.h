@@ -126,16 +126,35 @@ typedef struct ntk_gated_seam_desc {
 } ntk_gated_seam_desc;
 int ntk_gated_seam(const ntk_gated_seam_desc* d, void* stream);
 
+/* The seam of a layer whose sublayer results are RMS-normed and scaled before they join the stream, in one launch per row:
+ *   x[t] += mult * add_y[t] / sqrt(mean(add_y[t]^2) + eps) * add_w      (add_y may be NULL: nothing is owed)
+ *   h[t]  = x[t] / sqrt(mean(x[t]^2) + eps) * w                          (h may be NULL: no norm follows)
+ * Plain weights (nothing is added to them). */
+int ntk_rms_seam(float* h, int ldh, float* x, int ldx, const float* add_y, int ldy, const float* add_w, float mult, const float* w, int T, int n, float eps,
+                 void* stream);
+/* A short causal convolution over time on every channel, then an activation: y[t][c] = act(sum_j w[c][j] * in(t - (taps - 1) + j)[c]), w F32 [n][taps] (tap
+ * taps - 1 weighs the present token), in(.) = x rows of this portion, the carried inputs `state` [taps - 1][n] for the rows before it, zeros before the
+ * sequence's start (position pos0 + index < 0).  The portion's last taps - 1 inputs are left in `state`.  act 0: none, 1: silu.  y must not overlap x.
+ * 1 <= taps <= 16 (taps 1: no state is read or written). */
+int ntk_causal_conv_act(float* y, int ldy, const float* x, int ldx, const float* w, float* state, int taps, int act, int pos0, int T, int n, void* stream);
+/* x[t][i] = cap * tanh(x[t][i] / cap) over T rows of n */
+int ntk_softcap_rows(float* x, int ldx, float cap, int T, int n, void* stream);
+/* y[t][h][0..dv) *= sigmoid(g[t][h]): one gate per token and head (g rows ldg floats apart) */
+int ntk_head_gate(float* y, int ldy, const float* g, int ldg, int T, int H, int dv, void* stream);
+
 /* ---- latent_attention.hip ---------------------------------------------------------------------------------------------------------
  * Attention whose keys and values are up-projections of one cached latent per position plus one rotated key part shared by the heads.
  * The cache of a layer run holds rows of `row` = kv_rank + rot_dim floats: [latent (normed) | rotated key part].                       */
 typedef struct ntk_rotary {       /* angle of pair i at position p: p * freq[i]; cos and sin times mag */
     const double* freq;           /* device F64 [dims / 2] (after any frequency scaling): angles are formed in double, applied in F32 */
     float mag;
-    int dims;                     /* rotated entries at the head of the vector, neighbours (2i, 2i+1) paired */
+    int dims;                     /* rotated entries at the head of the vector */
+    int layout;                   /* NTK_ROT_NEIGHBOURS (0): entries (2i, 2i+1) form pair i; NTK_ROT_HALVES (1): entries (i, i + dims/2) do */
 } ntk_rotary;
+#define NTK_ROT_NEIGHBOURS 0
+#define NTK_ROT_HALVES 1
 /* For T tokens at positions pos0 ...: kv [T][ldkv] = [kv_rank raw latent | rot_dim raw key part] -> cache rows pos0 .. pos0+T-1:
- * latent / rms * norm_w, key part rotated (its first rot->dims entries; the rest copied).  q [T][H][qd], ldq floats between tokens: the rot_dim entries at the
+ * latent / rms * norm_w, key part rotated (its first rot->dims entries, paired by rot->layout; the rest copied).  q [T][H][qd], ldq floats between tokens: the rot_dim entries at the
  * end of every head rotated in place the same way. */
 int ntk_latent_prepare(float* cache, int row, const float* kv, int ldkv, const float* norm_w, float eps, int kv_rank, int rot_dim, float* q, int ldq, int H, int qd,
                        const ntk_rotary* rot, int pos0, int T, void* stream);
@@ -156,13 +175,16 @@ int ntk_latent_fold_query(float* qf, const float* q, int ldq, const void* w_uk, 
 /* out[t][h*dv + v] = sum_r W_uv[h*dv + v][r] * lat[t][h][r]  (the value up-projection applied after the weighted sum), times sigmoid(gate[t][h*dv+v]) if gate */
 int ntk_latent_unfold_value(float* out, int ldo, const float* lat, const void* w_uv, int wdtype, const float* gate, int ldg, int T, int H, int dv, int R,
                             void* stream);
+/* ... head_gate != 0: the gate is one number per token and head, gate[t][h] (ldg >= H) */
+int ntk_latent_unfold_value_ex(float* out, int ldo, const float* lat, const void* w_uv, int wdtype, const float* gate, int ldg, int head_gate, int T, int H, int dv,
+                               int R, void* stream);
 
 /* ---- window_attention.hip ---------------------------------------------------------------------------------------------------------
  * Grouped-query softmax attention over a cache of rotated keys and values, causal with an optional sliding window, with `maps` (1 or 2) score maps per
  * head that share the values.  Cache row of a position: [G][maps][dn] rotated keys | [G][dv] values (row >= G * (maps * dn + dv) floats).
  * Query head h uses key/value head h / (H / G); q [T][H][maps][dn].
- * ntk_window_prepare rotates q in place and k into the cache rows pos0 .. pos0+T-1 (the first rot->dims entries of every map of every head, neighbours
- * (2i, 2i+1) paired; the rest unchanged) and copies v behind the keys. */
+ * ntk_window_prepare rotates q in place and k into the cache rows pos0 .. pos0+T-1 (the first rot->dims entries of every map of every head, paired by
+ * rot->layout; the rest unchanged) and copies v behind the keys. */
 int ntk_window_prepare(float* cache, int row, float* q, int ldq, const float* k, int ldk, const float* v, int ldv, int H, int G, int maps, int dn, int dv,
                        const ntk_rotary* rot, int pos0, int T, void* stream);
 /* The same with what a projection leaves to its consumer: q = (q + qb) * (1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)) at position p before the
@@ -171,6 +193,21 @@ int ntk_window_prepare(float* cache, int row, float* q, int ldq, const float* k,
 int ntk_window_prepare_biased(float* cache, int row, float* q, int ldq, const float* k, int ldk, const float* v, int ldv, int H, int G, int maps, int dn, int dv,
                               const ntk_rotary* rot, const float* qb, const float* kb, const float* vb, float temp_coef, double temp_every, int pos0, int T,
                               void* stream);
+/* The general form.  Besides the above: values blended with another layer's values of the same tokens on their way into the cache rows,
+ * v <- (1 - v_blend) * v + v_blend * v_other[t] (v_other [T][G*dv], ld_other floats between tokens; NULL: no blending), and the values as the projection
+ * left them (+ vb) copied to v_keep [T][G*dv] (ld_keep; NULL: not kept) for a later layer to blend with. */
+typedef struct ntk_window_prepare_desc {
+    float* cache; int row;
+    float* q; int ldq; const float* k; int ldk; const float* v; int ldv;
+    int H, G, maps, dn, dv;
+    const ntk_rotary* rot;
+    const float* qb; const float* kb; const float* vb;
+    float temp_coef; double temp_every;
+    const float* v_other; int ld_other; float v_blend;
+    float* v_keep; int ld_keep;
+    int pos0, T;
+} ntk_window_prepare_desc;
+int ntk_window_prepare_ex(const ntk_window_prepare_desc* d, void* stream);
 /* a_m = softmax_j(scale * q_m . k_m[j]) V over the visible j (j <= p, and p - j < window if window > 0), per map m.
  * maps == 1: out = a_0.  maps == 2: out = a_0 - lambda * a_1 (a differential pair).  sub_norm != 0: out is then divided by sqrt(mean(out^2) + eps) over
  * the head's dv values.  out_scale multiplies the result.  out [T][H][dv], ldo floats between tokens.
@@ -187,7 +224,14 @@ typedef struct ntk_window_attention_desc {
     /* a learned bias by distance, added to the scaled score (not scaled itself): rel[bucket_of[min(p - j, n_dist - 1)] * H + h].
      * rel device F32 [buckets][H], bucket_of device int [n_dist].  rel == NULL: none. */
     const float* rel; const int* bucket_of; int n_dist;
+    /* mask_mode NTK_MASK_CHUNKS: `window` is a chunk size -- j is visible iff j <= p and floor(j / window) == floor(p / window), chunks counted from
+     * position 0 (NTK_MASK_SLIDING, 0: the sliding window above).
+     * softcap > 0: the scaled (and biased) score s becomes softcap * tanh(s / softcap).
+     * sink != 0: one more term exp(0) in the softmax's denominator (a key of score 0 that carries no value): p_j = exp(s_j) / (1 + sum exp(s)). */
+    int mask_mode; float softcap; int sink;
 } ntk_window_attention_desc;
+#define NTK_MASK_SLIDING 0
+#define NTK_MASK_CHUNKS 1
 size_t ntk_window_attention_scratch(int T, int H, int maps, int dv, int nkeys);
 int ntk_window_attention(const ntk_window_attention_desc* d, void* stream);
 
@@ -217,6 +261,7 @@ int ntk_lightning_attention(float* out, int ldo, const float* q, int ldq, const 
 #define NTK_DECAY_GIVEN 0
 #define NTK_DECAY_SIGMOID_ROOT 1
 #define NTK_DECAY_EXP_SIGMOID 2
+#define NTK_DECAY_EXP_SOFTPLUS 3
 typedef struct ntk_gated_recurrence_desc {
     float* out; int ldo;
     const float* q; int ldq;
@@ -228,11 +273,22 @@ typedef struct ntk_gated_recurrence_desc {
     int H, dn, dv;
     float q_scale;
     int pos0, T;
+    /* ---- the delta rule with one gate per head (all zero / NULL: the forms above) ----
+     * G > 0: q and k have G heads [T][G][dn] and state head h reads head h / (H / G) of them (H % G == 0).
+     * unit_q / unit_k != 0: q (before q_scale) / the written key k are divided by sqrt(sum x^2 + unit_eps) over the head's dn entries.
+     * head_gates != 0: wz and az hold ONE number per token and head ([T][H], ldw / lda >= H; wb, ab [H]): a decay and a removal rate for all channels.
+     * decay_form NTK_DECAY_EXP_SOFTPLUS: w = exp(-rate * softplus(z)), rate = decay_rates[h] (device F32 [H]) or decay_param where that is NULL.
+     * write_gated != 0 (needs az): the delta rule proper -- the removal is taken from the DECAYED state and the write is scaled by the removal rate:
+     *     S' = diag(w_t) S_(t-1),   S_t = S' - a_t u_t (u_t^T S') + a_t k_t v_t^T
+     * Any of these makes every portion form its vectors in a launch of its own: scratch must hold ntk_gated_recurrence_scratch_ex(d) floats. */
+    int G, unit_q, unit_k, head_gates, write_gated;
+    const float* decay_rates;
     float* scratch;   /* F32 [>= ntk_gated_recurrence_scratch(T, H, dn, dv, az != NULL)]: portions of more than a few tokens form their per-token vectors in a launch
                          of their own, once per head instead of once per workgroup, and long portions are walked in segments side by side (their states and
                          what the outputs are still owed are settled by two more launches); NULL: always inside the walk, tokens strictly in turn */
 } ntk_gated_recurrence_desc;
 size_t ntk_gated_recurrence_scratch(int T, int H, int dn, int dv, int removal);
+size_t ntk_gated_recurrence_scratch_ex(const ntk_gated_recurrence_desc* d);   /* from d's T, H, dn, dv, az and the per-head options */
 int ntk_gated_recurrence(const ntk_gated_recurrence_desc* d, void* stream);
 
 /* ---- moe.hip ---------------------------------------------------------------------------------------------------------------------- */

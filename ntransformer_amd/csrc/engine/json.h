@@ -36,6 +36,7 @@ public:
     const Json& at(const std::string& key) const { static const Json none; const Json* j = find(key); return j ? *j : none; }
     double number(double dflt = 0.0) const { return kind == NUM ? num : dflt; }
     long long integer(long long dflt = 0) const { return kind == NUM ? (long long)num : dflt; }
+    bool truth(bool dflt = false) const { return kind == BOOL ? b : kind == NUM ? num != 0.0 : dflt; }   // true / false (or a number that is not zero)
 
     // parse `n` bytes; on failure returns false and leaves *this null
     bool parse(const char* s, size_t n) {

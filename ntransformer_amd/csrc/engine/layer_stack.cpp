@@ -25,11 +25,18 @@ static StackForm gated_form() {
     f.gated = true; f.loop_projection = false;
     return f;
 }
+static StackForm scaled_form() {
+    StackForm f;
+    f.scaled = true; f.loop_projection = false;
+    f.mask_chunks = true; f.attention_sink = true; f.attention_gate = true; f.rot_halves = true; f.latent_head_gate = true;
+    return f;
+}
 // what the gated form's mechanisms fix
 static constexpr float kGeluAlpha = 1.5957691216057308f;   // 2 sqrt(2 / pi): 0.5 (1 + tanh y) = sigmoid(2 y)
 static constexpr float kGeluCubic = 0.044715f;
 static constexpr float kDeltaDecayRate = 0.6065306597126334f;   // exp(-1/2): w = exp(-rate * sigmoid(.))
 static constexpr float kUnitKeyEps = 1e-6f;
+static FamilyRegistrar reg_fifotar("Fifotar", [] { return std::unique_ptr<SequenceModel>(new LayerStackModel(scaled_form())); });
 static FamilyRegistrar reg_tubazen("Tubazen", [] { return std::unique_ptr<SequenceModel>(new LayerStackModel(gated_form())); });
 static FamilyRegistrar reg_fabolorn("Fabolorn", [] { return std::unique_ptr<SequenceModel>(new LayerStackModel(parallel_form())); });
 static FamilyRegistrar reg_nizorax("Nizorax", [] { return std::unique_ptr<SequenceModel>(new LayerStackModel(sequential_form())); });
@@ -96,6 +103,8 @@ int LayerStackModel::parse_mixer(const Json& L, const std::string& type, LatentM
         }
         m.rot_mag = (float)(0.1 * std::log(factor) + 1.0);
     }
+    m.rot_layout = form_.rot_halves ? NTK_ROT_HALVES : NTK_ROT_NEIGHBOURS;
+    m.head_gate = form_.latent_head_gate;
     m.rot_freq = (double*)dev_alloc(f.size() * sizeof(double));
     if (!m.rot_freq) return fail(NTK_E_NOMEM, "out of device memory");
     nt_hip_memcpy_h2d(m.rot_freq, f.data(), f.size() * sizeof(double));
@@ -136,6 +145,12 @@ int LayerStackModel::parse_window(const Json& L, WindowMixer& m) {
     m.diff = (float)mx.at("diff").number(0.0);
     m.window = 0;
     if (mx.has("mask") && !need_int(mx.at("mask"), "size", m.window, err_, where + " mask")) return NTK_E_FORMAT;
+    m.mask_mode = form_.mask_chunks ? NTK_MASK_CHUNKS : NTK_MASK_SLIDING;
+    m.sink = form_.attention_sink;
+    m.gated = form_.attention_gate;
+    m.softcap = (float)mx.at("softcap").number(0.0);
+    if (m.softcap < 0.0f) return fail(NTK_E_FORMAT, where + ": 'softcap' must be positive");
+    m.v_mix = form_.scaled && mx.at("v_mix").truth();
     m.rot_dims = 0;
     std::vector<double> f(1, 0.0);
     if (mx.has("rot")) {
@@ -183,6 +198,21 @@ int LayerStackModel::parse_gla(const Json& L, GlaMixer& m) {
     return NTK_OK;
 }
 
+int LayerStackModel::parse_gated_delta(const Json& L, GatedDeltaMixer& m) {
+    const Json& mx = L.at("mixer");
+    const std::string where = "mixer 'delta'";
+    if (!mx.is_object()) return fail(NTK_E_FORMAT, where + ": no 'mixer' object");
+    if (!need_int(mx, "heads", m.heads, err_, where) || !need_int(mx, "dim", m.dim, err_, where) || !need_int(mx, "vdim", m.vdim, err_, where)) return NTK_E_FORMAT;
+    m.kv_heads = m.heads;
+    if (mx.has("kv_heads") && !need_int(mx, "kv_heads", m.kv_heads, err_, where)) return NTK_E_FORMAT;
+    if (m.heads % m.kv_heads) return fail(NTK_E_FORMAT, where + ": heads must be a multiple of kv_heads");
+    m.taps = 1;
+    if (mx.has("conv") && !need_int(mx, "conv", m.taps, err_, where)) return NTK_E_FORMAT;
+    if (m.taps > 16) return fail(NTK_E_SHAPE, where + ": convolutions of up to 16 taps are supported");
+    if (m.dim > 1024 || m.vdim > 1024) return fail(NTK_E_SHAPE, where + ": dim and vdim up to 1024 are supported");
+    return NTK_OK;
+}
+
 int LayerStackModel::parse_parallel(const Json& L, ParallelMixer& m) {
     const Json& mx = L.at("mixer");
     const std::string where = "mixer 'parallel'";
@@ -214,12 +244,19 @@ int LayerStackModel::parse_parallel(const Json& L, ParallelMixer& m) {
 
 int LayerStackModel::parse_mlp(const Json& ml, const std::string& where, StackLayer& S) {
     const std::string kind = ml.at("kind").is_string() ? ml.at("kind").str : "moe";
+    if (kind == "dense" && form_.scaled) {
+        S.mlp_kind = kMlpClipped;
+        if (!need_int(ml, "ff", S.cff.ff, err_, where)) return NTK_E_FORMAT;
+        S.cff.limit = ml.at("limit").is_number() ? (float)ml.at("limit").number() : INFINITY;
+        if (!(S.cff.limit > 0.0f)) return fail(NTK_E_FORMAT, where + ": 'limit' must be positive");
+        return NTK_OK;
+    }
     if (kind == "dense") {
         S.mlp_kind = kMlpDense;
         if (!need_int(ml, "ff", form_.gated ? S.gff.ff : S.ffn.ff, err_, where)) return NTK_E_FORMAT;
         return NTK_OK;
     }
-    if (form_.gated) return fail(NTK_E_FORMAT, where + ": this family has the dense feed-forward only");
+    if (form_.gated || form_.scaled) return fail(NTK_E_FORMAT, where + ": this family has the dense feed-forward only");
     if (kind != "moe") return fail(NTK_E_FORMAT, where + ": unknown kind '" + kind + "'");
     S.mlp_kind = kMlpMoe;
     MoeFeedForward& M = S.mlp;
@@ -262,6 +299,13 @@ int LayerStackModel::parse(const ModelFolder& f) {
         logit_scale_ = (float)c.at("logit_scale").number(1.0);
         has_state_ = true;
     }
+    if (form_.scaled) {
+        embed_scale_ = (float)c.at("embedding").at("scale").number(1.0);
+        residual_mult_ = (float)c.at("residual_mult").number(1.0);
+        logit_softcap_ = (float)c.at("logit_softcap").number(0.0);
+        if (logit_softcap_ < 0.0f) return fail(NTK_E_FORMAT, "config: logit_softcap must be positive");
+        norm_offset_ = 0.0f;
+    }
     if (c.at("bos").is_number()) info_.bos = (int)c.at("bos").integer();
     if (c.at("eos").is_number()) info_.eos = (int)c.at("eos").integer();
     const Json& ls = c.at("layers");
@@ -272,7 +316,11 @@ int LayerStackModel::parse(const ModelFolder& f) {
         StackLayer& S = layers_[i];
         S.type = L.at("type").str;
         // which mixers a form lists: the parallel form's layers read two norms of one input, so its mixers are the latent kinds it was built around
-        if (form_.gated && S.type == "gla") { S.mixer = kMixGla; LS_TRY(parse_gla(L, S.gla)); }
+        if (form_.scaled && S.type == "attention") { S.mixer = kMixWindow; LS_TRY(parse_window(L, S.att)); }
+        else if (form_.scaled && S.type == "latent_attention") { S.mixer = kMixLatent; LS_TRY(parse_mixer(L, S.type, S.mix)); }
+        else if (form_.scaled && S.type == "delta") { S.mixer = kMixGatedDelta; LS_TRY(parse_gated_delta(L, S.gdl)); has_state_ = true; }
+        else if (form_.scaled) return fail(NTK_E_FORMAT, "layer " + std::to_string(i) + ": unknown mixer type '" + S.type + "'");
+        else if (form_.gated && S.type == "gla") { S.mixer = kMixGla; LS_TRY(parse_gla(L, S.gla)); }
         else if (form_.gated && S.type == "parallel") { S.mixer = kMixParallel; LS_TRY(parse_parallel(L, S.par)); }
         else if (form_.gated) return fail(NTK_E_FORMAT, "layer " + std::to_string(i) + ": unknown mixer type '" + S.type + "'");
         else if (!form_.sequential && (S.type == "latent_attention" || S.type == "latent_attention_2")) { S.mixer = kMixLatent; LS_TRY(parse_mixer(L, S.type, S.mix)); }
@@ -281,12 +329,20 @@ int LayerStackModel::parse(const ModelFolder& f) {
         else return fail(NTK_E_FORMAT, "layer " + std::to_string(i) + ": unknown mixer type '" + S.type + "'");
         S.has_mlp = L.has("mlp") && !L.at("mlp").is_null();
         if (S.has_mlp) LS_TRY(parse_mlp(L.at("mlp"), "layer " + std::to_string(i) + " mlp", S));
-        if (!form_.sequential && !form_.gated && S.mlp_kind == kMlpDense) return fail(NTK_E_FORMAT, "layer " + std::to_string(i) + ": this family has no dense feed-forward");
+        if (!form_.sequential && !form_.gated && !form_.scaled && S.mlp_kind == kMlpDense) return fail(NTK_E_FORMAT, "layer " + std::to_string(i) + ": this family has no dense feed-forward");
     }
     // the order of layer runs
     const int n = (int)layers_.size();
     runs_.clear();
-    has_loop_ = c.has("loop") && !form_.gated;   // (the gated form's depth weights are per layer: it has no repeated span)
+    has_loop_ = c.has("loop") && !form_.gated && !form_.scaled;   // (the gated form's depth weights are per layer: it has no repeated span; the scaled form lists none)
+    if (form_.scaled) {   // values are blended with those of the FIRST blending attention layer, which therefore only keeps its own
+        const WindowMixer* first = nullptr;
+        for (auto& S : layers_) {
+            if (S.mixer != kMixWindow || !S.att.v_mix) continue;
+            if (!first) { S.att.v_source = true; first = &S.att; continue; }
+            if (S.att.kv_heads * S.att.vdim != first->kv_heads * first->vdim) return fail(NTK_E_FORMAT, "config: attention layers that blend their values must have the same kv_heads * vdim");
+        }
+    }
     if (has_loop_) {
         const Json& lp = c.at("loop");
         const int a = (int)lp.at("start").integer(), b = (int)lp.at("stop").integer(), times = (int)lp.at("times").integer(1);
@@ -498,10 +554,15 @@ int LayerStackModel::upload_mixer(const ModelFolder& f, const std::string& p, in
     const std::string li = "layer " + std::to_string(i);
     if (L.mixer == kMixWindow) {
         WindowMixer& m = L.att;
-        LS_TRY(upload_matrix(f, {p + "mix.q", p + "mix.k", p + "mix.v"}, W, m.in));
+        if (m.gated) LS_TRY(upload_matrix(f, {p + "mix.q", p + "mix.k", p + "mix.v", p + "mix.g"}, W, m.in));
+        else LS_TRY(upload_matrix(f, {p + "mix.q", p + "mix.k", p + "mix.v"}, W, m.in));
         m.k_off = m.heads * m.maps * m.dim;
         m.v_off = m.k_off + m.kv_heads * m.maps * m.dim;
-        if (m.in.out_f != m.v_off + m.kv_heads * m.vdim) return fail(NTK_E_SHAPE, li + ": the mixer's input projections do not have the configured sizes");
+        m.g_off = m.v_off + m.kv_heads * m.vdim;
+        const StTensor* tk = f.tensor(p + "mix.k");
+        if (!tk || tk->shape[0] != m.v_off - m.k_off) return fail(NTK_E_SHAPE, "tensor '" + p + "mix.k' does not have kv_heads * maps * dim rows");
+        if (m.v_mix && !m.v_source) LS_TRY(read_scalar(f, p + "mix.vmix", &m.v_blend));
+        if (m.in.out_f != m.g_off + (m.gated ? m.heads * m.vdim : 0)) return fail(NTK_E_SHAPE, li + ": the mixer's input projections do not have the configured sizes");
         const StTensor* tq = f.tensor(p + "mix.q");
         if (!tq || tq->shape[0] != m.k_off) return fail(NTK_E_SHAPE, "tensor '" + p + "mix.q' does not have heads * maps * dim rows");
         LS_TRY(upload_matrix(f, {p + "mix.o"}, (int64_t)m.heads * m.vdim, m.o));
@@ -539,6 +600,46 @@ int LayerStackModel::upload_mixer(const ModelFolder& f, const std::string& p, in
         if (m.o.out_f != W) return fail(NTK_E_SHAPE, "tensor '" + p + "mix.o' does not have 'width' rows");
         return NTK_OK;
     }
+    if (L.mixer == kMixGatedDelta) {
+        GatedDeltaMixer& m = L.gdl;
+        const int gq = m.kv_heads * m.dim, hv = m.heads * m.vdim, nc = m.channels();
+        LS_TRY(upload_matrix(f, {p + "mix.q", p + "mix.k", p + "mix.v", p + "mix.g", p + "mix.b", p + "mix.a"}, W, m.in));
+        m.k_off = gq; m.v_off = 2 * gq; m.g_off = nc; m.b_off = nc + hv; m.a_off = m.b_off + m.heads;
+        auto rows_of = [&](const std::string& nm) -> int64_t { const StTensor* t = f.tensor(nm); return t && t->shape.size() == 2 ? t->shape[0] : -1; };
+        if (rows_of(p + "mix.q") != gq || rows_of(p + "mix.k") != gq || rows_of(p + "mix.v") != hv || rows_of(p + "mix.g") != hv || rows_of(p + "mix.b") != m.heads ||
+            rows_of(p + "mix.a") != m.heads)
+            return fail(NTK_E_SHAPE, li + ": the mixer's input projections do not have the configured sizes");
+        // the three convolutions one below the other, like their channels in the product's result
+        std::vector<float> cw((size_t)nc * m.taps);
+        size_t at = 0;
+        for (const char* nm : {"mix.q.conv", "mix.k.conv", "mix.v.conv"}) {
+            const StTensor* t = f.tensor(p + nm);
+            if (!t) return fail(NTK_E_FORMAT, "tensor '" + p + nm + "' is missing");
+            if (t->shape.size() != 2 || t->shape[1] != m.taps || at + (size_t)t->numel() > cw.size()) return fail(NTK_E_SHAPE, "tensor '" + p + nm + "' is not [channels, conv]");
+            if (!tensor_to_f32(*t, cw.data() + at)) return fail(NTK_E_DTYPE, "tensor '" + p + nm + "': dtype " + t->dtype + " is not supported");
+            at += (size_t)t->numel();
+            weight_bytes_ += t->nbytes;
+        }
+        if (at != cw.size()) return fail(NTK_E_SHAPE, li + ": the convolutions do not cover the channels of q, k and v");
+        m.conv = (float*)dev_alloc(cw.size() * sizeof(float));
+        if (!m.conv) return fail(NTK_E_NOMEM, "out of device memory");
+        nt_hip_memcpy_h2d(m.conv, cw.data(), cw.size() * sizeof(float));
+        // rate = exp(A_log), in F32
+        const StTensor* al = f.tensor(p + "mix.A_log");
+        if (!al || al->numel() != m.heads) return fail(NTK_E_SHAPE, "tensor '" + p + "mix.A_log' does not have one entry per head");
+        std::vector<float> rate((size_t)m.heads);
+        if (!tensor_to_f32(*al, rate.data())) return fail(NTK_E_DTYPE, "tensor '" + p + "mix.A_log': dtype " + al->dtype + " is not supported");
+        for (auto& r : rate) r = std::exp(r);
+        weight_bytes_ += al->nbytes;
+        m.rates = (float*)dev_alloc(rate.size() * sizeof(float));
+        if (!m.rates) return fail(NTK_E_NOMEM, "out of device memory");
+        nt_hip_memcpy_h2d(m.rates, rate.data(), rate.size() * sizeof(float));
+        LS_TRY(upload_vector(f, p + "mix.dt_bias", m.heads, &m.dt_bias));
+        LS_TRY(upload_vector(f, p + "mix.norm", m.vdim, &m.norm));
+        LS_TRY(upload_matrix(f, {p + "mix.o"}, hv, m.o));
+        if (m.o.out_f != W) return fail(NTK_E_SHAPE, "tensor '" + p + "mix.o' does not have 'width' rows");
+        return NTK_OK;
+    }
     LatentMixer& m = L.mix;
     const int hq = m.heads * m.qd(), hv = m.heads * m.vdim;
     const std::string first = m.q_rank ? p + "mix.dq" : p + "mix.q";
@@ -546,7 +647,7 @@ int LayerStackModel::upload_mixer(const ModelFolder& f, const std::string& p, in
     m.q_off = 0;
     m.kv_off = m.q_rank ? m.q_rank : hq;
     m.g_off = m.kv_off + m.row();
-    if (m.in.out_f != m.g_off + hv) return fail(NTK_E_SHAPE, li + ": the mixer's input projections do not have the configured sizes");
+    if (m.in.out_f != m.g_off + (m.head_gate ? m.heads : hv)) return fail(NTK_E_SHAPE, li + ": the mixer's input projections do not have the configured sizes");
     if (m.q_rank) {
         LS_TRY(upload_vector(f, p + "mix.dq.norm", m.q_rank, &m.q_norm));
         LS_TRY(upload_matrix(f, {p + "mix.uq"}, m.q_rank, m.uq));
@@ -563,6 +664,14 @@ int LayerStackModel::upload_mixer(const ModelFolder& f, const std::string& p, in
 int LayerStackModel::upload_mlp(const ModelFolder& f, const std::string& p, int i, StackLayer& L) {
     const int W = info_.width;
     const std::string li = "layer " + std::to_string(i);
+    if (L.mlp_kind == kMlpClipped) {
+        GatedExperts& D = L.cff;
+        LS_TRY(upload_matrix(f, {p + "mlp.gate", p + "mlp.up"}, W, D.gate_up));
+        LS_TRY(upload_matrix(f, {p + "mlp.down"}, D.ff, D.down));
+        const StTensor* tg = f.tensor(p + "mlp.gate");
+        if (D.gate_up.out_f != 2 * D.ff || !tg || tg->shape[0] != D.ff || D.down.out_f != W) return fail(NTK_E_SHAPE, li + ": feed-forward matrices do not have the configured sizes");
+        return NTK_OK;
+    }
     if (L.mlp_kind == kMlpDense) {
         DenseFeedForward& D = L.ffn;
         LS_TRY(upload_matrix(f, {p + "mlp.up"}, W, D.up));
@@ -611,9 +720,11 @@ int LayerStackModel::upload_layer(const ModelFolder& f, int i, StackLayer& L) {
         LS_TRY(upload_norm(f, p + "norm1b", L.norm1b));
         LS_TRY(upload_vector(f, p + "canon1", (int64_t)W * taps_, &L.canon1));
     }
+    if (form_.scaled) LS_TRY(upload_norm(f, p + "norm1b", L.norm1b));
     LS_TRY(upload_mixer(f, p, i, L));
     if (L.has_mlp) {
         LS_TRY(upload_norm(f, p + "norm2", L.norm2));
+        if (form_.scaled) LS_TRY(upload_norm(f, p + "norm2b", L.norm2b));
         if (form_.sequential) {
             LS_TRY(upload_norm(f, p + "norm2b", L.norm2b));
             LS_TRY(upload_vector(f, p + "canon2", (int64_t)W * taps_, &L.canon2));
@@ -636,7 +747,8 @@ int LayerStackModel::load(const std::string& dir, const SeqLoadOptions& opt) {
     LS_TRY(parse(f));
     const int W = info_.width;
     LS_TRY(upload_matrix(f, {"embed"}, W, embed_));
-    LS_TRY(upload_matrix(f, {"head"}, W, head_));
+    if (form_.scaled) head_ = embed_;   // the embedding table itself (without the embedding's scale) is the head
+    else LS_TRY(upload_matrix(f, {"head"}, W, head_));
     if (embed_.out_f != info_.vocab || head_.out_f != info_.vocab) return fail(NTK_E_SHAPE, "embed / head do not have 'vocab' rows");
     LS_TRY(upload_norm(f, "final.norm", final_norm_));
     if (form_.gated) {
@@ -677,11 +789,20 @@ int LayerStackModel::alloc_buffers() {
             max_hr_ = std::max(max_hr_, m.heads * m.kv_rank);
             if (m.kv_rank > 512 || m.vdim > 512) return fail(NTK_E_SHAPE, "kv_rank and vdim up to 512 are supported");
             sc = std::max(sc, ntk_latent_attention_scratch(kSharedRows, m.heads, m.kv_rank, opt_.max_context));
+        } else if (L.mixer == kMixGatedDelta) {
+            const GatedDeltaMixer& m = L.gdl;
+            max_in_ = std::max<int>(max_in_, (int)m.in.out_f);
+            max_hdv_ = std::max(max_hdv_, m.heads * m.vdim);
+            max_conv_ = std::max(max_conv_, m.channels());
+            ntk_gated_recurrence_desc d{};
+            d.T = chunk_; d.H = m.heads; d.dn = m.dim; d.dv = m.vdim; d.az = (const float*)&d; d.head_gates = 1; d.write_gated = 1;   // (az: only whether there is a removal term is looked at)
+            rsc = std::max(rsc, ntk_gated_recurrence_scratch_ex(&d));
         } else if (L.mixer == kMixWindow) {
             const WindowMixer& m = L.att;
             max_in_ = std::max<int>(max_in_, (int)m.in.out_f);
             max_hdv_ = std::max(max_hdv_, m.heads * m.vdim);
             if (m.vdim > 512) return fail(NTK_E_SHAPE, "vdim up to 512 is supported");
+            if (m.v_mix) max_gv_ = std::max(max_gv_, m.kv_heads * m.vdim);
             wsc = std::max(wsc, ntk_window_attention_scratch(chunk_, m.heads, m.maps, m.vdim, opt_.max_context));
         } else if (L.mixer == kMixLightning) {
             const LightningMixer& m = L.lin;
@@ -710,6 +831,8 @@ int LayerStackModel::alloc_buffers() {
             if (L.mlp.has_shared) max_sff2_ = std::max(max_sff2_, 2 * L.mlp.shared.ff);
         } else if (L.mlp_kind == kMlpDense && !form_.gated) {
             max_ffn_ = std::max(max_ffn_, L.ffn.ff);
+        } else if (L.mlp_kind == kMlpClipped) {
+            max_ffn_ = std::max(max_ffn_, L.cff.ff);
         }
     }
     const size_t C = (size_t)chunk_, ctx = (size_t)opt_.max_context;
@@ -724,6 +847,9 @@ int LayerStackModel::alloc_buffers() {
     if (form_.gated)
         ok = ok && fl(&ff_, C * W) && fl(&zf_, C * max_ffn_) && fl(&wscratch_, wsc) && fl(&results_, (runs_.size() + 1) * C * W) && fl(&zq_, C * std::max(max_rec_, 1)) && fl(&rscratch_, rsc) &&
              fl(&gu2_, C * std::max(max_gu2_, 1));
+    if (form_.scaled)
+        ok = ok && fl(&ff_, C * W) && fl(&zf_, C * std::max(max_ffn_, 1)) && fl(&gu2_, C * 2 * std::max(max_ffn_, 1)) && fl(&wscratch_, wsc) && fl(&rscratch_, rsc) &&
+             fl(&cv_, C * std::max(max_conv_, 1)) && fl(&vfirst_, C * std::max(max_gv_, 1));
     want_dev_ = tokens_dev_ ? tokens_dev_ + C : nullptr;   // one staging area: [tokens of a pass | wanted places], filled by ONE stream-ordered copy from pinned memory
     h_stage_ = (int*)nt_hip_malloc_host(2 * C * sizeof(int));
     ok = ok && h_stage_ != nullptr;
@@ -766,14 +892,15 @@ int LayerStackModel::truncate_slot(int slot, int length) {
 }
 
 // ------------------------------------------------------------------------------------------------------------------------ the step
-int LayerStackModel::run_mixer(const StackLayer& L, float* cache, int T, int pos0) {
+int LayerStackModel::run_mixer(const StackLayer& L, float* cache, int T, int pos0, bool normed_input) {
     const LatentMixer& m = L.mix;
     const int W = info_.width, H = m.heads, qd = m.qd(), row = m.row(), hv = H * m.vdim, na = (int)m.in.out_f;
     // one product for [query (latent) | latent + key part | gate]; decoding: the layer's first norm and the query latent's norm run inside the products
+    // (normed_input: h1_ holds the normed stream already -- the seam in front of the mixer wrote it)
     const bool few = T <= ntk_dense_few_rows();
     ntk_dense_desc d{};
-    d.Y = a_; d.ldy = na; d.X = few ? x_ : h1_; d.ldx = W; d.W = m.in.ptr; d.wdtype = m.in.dtype; d.G = 1; d.row_div = 1; d.T = T; d.N = na; d.K = W;
-    if (few) { d.norm_w = L.norm1.w; d.norm_eps = eps_; d.norm_offset = 1.0f; }
+    d.Y = a_; d.ldy = na; d.X = few && !normed_input ? x_ : h1_; d.ldx = W; d.W = m.in.ptr; d.wdtype = m.in.dtype; d.G = 1; d.row_div = 1; d.T = T; d.N = na; d.K = W;
+    if (few && !normed_input) { d.norm_w = L.norm1.w; d.norm_eps = eps_; d.norm_offset = norm_offset_; }
     LS_TRY(ntk_dense(&d, stream_));
     float* q = a_;
     int ldq = na;
@@ -785,13 +912,13 @@ int LayerStackModel::run_mixer(const StackLayer& L, float* cache, int T, int pos
         q = q_;
         ldq = H * qd;
     }
-    ntk_rotary rot{m.rot_freq, m.rot_mag, m.rot_dims};
+    ntk_rotary rot{m.rot_freq, m.rot_mag, m.rot_dims, m.rot_layout};
     LS_TRY(ntk_latent_prepare(cache, row, a_ + m.kv_off, na, m.kv_norm, eps_, m.kv_rank, m.rot_dim, q, ldq, H, qd, &rot, pos0, T, stream_));
     if (T <= kSharedRows) {
         LS_TRY(ntk_latent_fold_query(qf_, q, ldq, m.uk.ptr, m.uk.dtype, T, H, m.dim, m.rot_dim, m.kv_rank, stream_));
         LS_TRY(ntk_latent_attention(lat_, H * m.kv_rank, qf_, H * row, nullptr, 0, nullptr, 0, cache, row, m.kv_rank, m.rot_dim, H, m.dim, m.vdim, 1, pos0, T, 0,
                                     m.window, m.scale, scratch_, stream_));
-        LS_TRY(ntk_latent_unfold_value(att_, hv, lat_, m.uv.ptr, m.uv.dtype, a_ + m.g_off, na, T, H, m.vdim, m.kv_rank, stream_));
+        LS_TRY(ntk_latent_unfold_value_ex(att_, hv, lat_, m.uv.ptr, m.uv.dtype, a_ + m.g_off, na, m.head_gate ? 1 : 0, T, H, m.vdim, m.kv_rank, stream_));
     } else {
         const int key0 = m.window > 0 ? std::max(0, pos0 - m.window + 1) : 0;
         const int nkeys = pos0 + T - key0;
@@ -799,7 +926,8 @@ int LayerStackModel::run_mixer(const StackLayer& L, float* cache, int T, int pos
         LS_TRY(ntk_dense_linear(vx_, hv, cache + (size_t)key0 * row, row, m.uv.ptr, m.uv.dtype, nkeys, hv, m.kv_rank, 0, stream_));
         LS_TRY(ntk_latent_attention(att_, hv, q, ldq, kx_, H * m.dim, vx_, hv, cache, row, m.kv_rank, m.rot_dim, H, m.dim, m.vdim, 0, pos0, T, key0, m.window, m.scale,
                                     nullptr, stream_));
-        LS_TRY(ntk_sigmoid_gate(att_, hv, a_ + m.g_off, na, T, hv, stream_));
+        if (m.head_gate) LS_TRY(ntk_head_gate(att_, hv, a_ + m.g_off, na, T, H, m.vdim, stream_));
+        else LS_TRY(ntk_sigmoid_gate(att_, hv, a_ + m.g_off, na, T, hv, stream_));
     }
     return ntk_dense_linear(mix_, W, att_, hv, m.o.ptr, m.o.dtype, T, W, hv, 0, stream_);
 }
@@ -809,14 +937,21 @@ int LayerStackModel::run_window(const StackLayer& L, float* cache, int T, int po
     const WindowMixer& m = L.att;
     const int W = info_.width, na = (int)m.in.out_f, hv = m.heads * m.vdim;
     LS_TRY(ntk_dense_linear(a_, na, h1_, W, m.in.ptr, m.in.dtype, T, na, W, 0, stream_));
-    ntk_rotary rot{m.rot_freq, 1.0f, m.rot_dims};
-    LS_TRY(ntk_window_prepare(cache, m.row(), a_, na, a_ + m.k_off, na, a_ + m.v_off, na, m.heads, m.kv_heads, m.maps, m.dim, m.vdim, &rot, pos0, T, stream_));
+    ntk_rotary rot{m.rot_freq, 1.0f, m.rot_dims, form_.rot_halves ? NTK_ROT_HALVES : NTK_ROT_NEIGHBOURS};
+    ntk_window_prepare_desc pd{};
+    pd.cache = cache; pd.row = m.row(); pd.q = a_; pd.ldq = na; pd.k = a_ + m.k_off; pd.ldk = na; pd.v = a_ + m.v_off; pd.ldv = na;
+    pd.H = m.heads; pd.G = m.kv_heads; pd.maps = m.maps; pd.dn = m.dim; pd.dv = m.vdim; pd.rot = &rot; pd.temp_every = 1.0; pd.pos0 = pos0; pd.T = T;
+    if (m.v_mix && m.v_source) { pd.v_keep = vfirst_; pd.ld_keep = m.kv_heads * m.vdim; }                 // the first blending layer keeps its values of this pass's tokens
+    else if (m.v_mix) { pd.v_other = vfirst_; pd.ld_other = m.kv_heads * m.vdim; pd.v_blend = m.v_blend; }    // the later ones blend with them
+    LS_TRY(ntk_window_prepare_ex(&pd, stream_));
     ntk_window_attention_desc d{};
     d.out = att_; d.ldo = hv; d.q = a_; d.ldq = na; d.cache = cache; d.row = m.row(); d.H = m.heads; d.G = m.kv_heads; d.maps = m.maps; d.dn = m.dim; d.dv = m.vdim;
     d.pos0 = pos0; d.T = T; d.window = m.window; d.scale = m.scale; d.lambda = m.lambda;
     d.sub_norm = m.maps == 2 ? 1 : 0; d.eps = eps_; d.out_scale = m.maps == 2 ? 1.0f - m.diff : 1.0f;
     d.scratch = wscratch_;
+    d.mask_mode = m.mask_mode; d.softcap = m.softcap; d.sink = m.sink ? 1 : 0;
     LS_TRY(ntk_window_attention(&d, stream_));
+    if (m.gated) LS_TRY(ntk_sigmoid_gate(att_, hv, a_ + m.g_off, na, T, hv, stream_));
     return ntk_dense_linear(mix_, W, att_, hv, m.o.ptr, m.o.dtype, T, W, hv, 0, stream_);
 }
 
@@ -830,18 +965,18 @@ int LayerStackModel::run_lightning(const StackLayer& L, float* state, int T, int
     return ntk_dense_linear(mix_, W, att_, hv, m.o.ptr, m.o.dtype, T, W, hv, 0, stream_);
 }
 
-int LayerStackModel::run_experts(const MoeFeedForward& M, const GatedExperts& ex, const float* h, float* gu, float* act, float* out, int rows, const int* offsets, const int* order, int top) {
+int LayerStackModel::run_experts(float glu_alpha, float glu_up_offset, const GatedExperts& ex, const float* h, float* gu, float* act, float* out, int rows, const int* offsets, const int* order, int top) {
     const int W = info_.width;
     ntk_dense_desc d{};
     d.Y = gu; d.ldy = 2 * ex.ff; d.X = h; d.ldx = W; d.W = ex.gate_up.ptr; d.wstride = ex.gate_up.stride(); d.wdtype = ex.gate_up.dtype;
     d.offsets = offsets; d.G = ex.gate_up.count; d.rows = order; d.row_div = top; d.T = rows; d.N = 2 * ex.ff; d.K = W; d.accumulate = 0;
     if (rows <= ntk_dense_few_rows()) {   // decoding: the activation inside the product's launch
-        d.Y = act; d.ldy = ex.ff; d.glu_ff = ex.ff; d.glu_limit = ex.limit; d.glu_alpha = M.glu_alpha; d.glu_up_offset = M.glu_up_offset;
+        d.Y = act; d.ldy = ex.ff; d.glu_ff = ex.ff; d.glu_limit = ex.limit; d.glu_alpha = glu_alpha; d.glu_up_offset = glu_up_offset;
         LS_TRY(ntk_dense(&d, stream_));
         d.glu_ff = 0;
     } else {
         LS_TRY(ntk_dense(&d, stream_));
-        LS_TRY(ntk_glu(act, gu, rows, ex.ff, ex.limit, M.glu_alpha, M.glu_up_offset, stream_));
+        LS_TRY(ntk_glu(act, gu, rows, ex.ff, ex.limit, glu_alpha, glu_up_offset, stream_));
     }
     d.Y = out; d.ldy = W; d.X = act; d.ldx = ex.ff; d.W = ex.down.ptr; d.wstride = ex.down.stride(); d.wdtype = ex.down.dtype;
     d.rows = nullptr; d.row_div = 1; d.N = W; d.K = ex.ff;
@@ -856,8 +991,8 @@ int LayerStackModel::run_moe(const StackLayer& L, int T, bool into_stream) {
     float* sgate = M.has_shared && M.shared_gate ? sg_ : nullptr;
     LS_TRY(ntk_moe_route_ex(ids_, wts_, sgate, h2_, W, M.router, sgate ? M.shared_gate : nullptr, T, W, M.experts, M.top, &M.route, stream_));
     LS_TRY(ntk_moe_group(offsets_, order_, where_, ids_, T, M.top, M.experts, stream_));
-    LS_TRY(run_experts(M, M.routed, h2_, gu_, act_, dn_, T * M.top, offsets_, order_, M.top));
-    if (M.has_shared) LS_TRY(run_experts(M, M.shared, h2_, sgu_, sact_, sdn_, T, nullptr, nullptr, 1));
+    LS_TRY(run_experts(M.glu_alpha, M.glu_up_offset, M.routed, h2_, gu_, act_, dn_, T * M.top, offsets_, order_, M.top));
+    if (M.has_shared) LS_TRY(run_experts(M.glu_alpha, M.glu_up_offset, M.shared, h2_, sgu_, sact_, sdn_, T, nullptr, nullptr, 1));
     if (into_stream) return ntk_moe_combine(x_, mix_, dn_, where_, wts_, M.has_shared ? sdn_ : nullptr, sgate, T, M.top, W, stream_);
     return ntk_moe_sum(ff_, dn_, where_, wts_, M.has_shared ? sdn_ : nullptr, sgate, T, M.top, W, stream_);
 }
@@ -869,6 +1004,51 @@ int LayerStackModel::run_dense_ff(const StackLayer& L, int T) {
     LS_TRY(ntk_dense_linear(zf_, D.ff, h2_, W, D.up.ptr, D.up.dtype, T, D.ff, W, 0, stream_));
     LS_TRY(ntk_polynorm(zf_, D.ff, zf_, D.ff, D.act, T, D.ff, eps_, stream_));
     return ntk_dense_linear(ff_, W, zf_, D.ff, D.down.ptr, D.down.dtype, T, W, D.ff, 0, stream_);
+}
+
+// the dense clipped gated unit (the experts' unit with one member): gate and up in one product (decoding: the activation inside its launch), down -> ff_
+int LayerStackModel::run_clipped_ff(const StackLayer& L, int T) {
+    return run_experts(kGluAlpha, 1.0f, L.cff, h2_, gu2_, zf_, ff_, T, nullptr, nullptr, 1);
+}
+
+// the delta rule with per-head gates: one product for [q | k | v | gate | beta | decay], the short convolutions of q, k and v (+ silu) with their carried
+// inputs, the recurrence (unit q and k, decay and write strength formed from their raw projections in its pre-pass), unit norm per head with the shared
+// weight and the silu gate, output projection -> mix_.  state = [S | the convolutions' last inputs]
+int LayerStackModel::run_gated_delta(const StackLayer& L, float* state, int T, int pos0) {
+    const GatedDeltaMixer& m = L.gdl;
+    const int W = info_.width, na = (int)m.in.out_f, nc = m.channels(), hv = m.heads * m.vdim;
+    LS_TRY(ntk_dense_linear(a_, na, h1_, W, m.in.ptr, m.in.dtype, T, na, W, 0, stream_));
+    LS_TRY(ntk_causal_conv_act(cv_, nc, a_, na, m.conv, state + m.recurrent_floats(), m.taps, 1, pos0, T, nc, stream_));
+    ntk_gated_recurrence_desc d{};
+    d.out = att_; d.ldo = hv; d.q = cv_; d.ldq = nc; d.k = cv_ + m.k_off; d.ldk = nc; d.v = cv_ + m.v_off; d.ldv = nc;
+    d.wz = a_ + m.a_off; d.ldw = na; d.wb = m.dt_bias; d.decay_form = NTK_DECAY_EXP_SOFTPLUS; d.decay_rates = m.rates;
+    d.az = a_ + m.b_off; d.lda = na; d.unit_eps = kUnitKeyEps;
+    d.G = m.kv_heads; d.unit_q = 1; d.unit_k = 1; d.head_gates = 1; d.write_gated = 1;
+    d.state = state; d.H = m.heads; d.dn = m.dim; d.dv = m.vdim; d.q_scale = 1.0f / std::sqrt((float)m.dim); d.pos0 = pos0; d.T = T; d.scratch = rscratch_;
+    LS_TRY(ntk_gated_recurrence(&d, stream_));
+    LS_TRY(ntk_head_rmsnorm_gate(att_, hv, att_, hv, m.norm, 0, a_ + m.g_off, na, 2, 1.0f, T, m.heads, m.vdim, eps_, stream_));
+    return ntk_dense_linear(mix_, W, att_, hv, m.o.ptr, m.o.dtype, T, W, hv, 0, stream_);
+}
+
+// the seam in front of a sublayer of the scaled form: what the stream is still owed joins it (RMS norm, weight, the residual factor), then the norm of the row
+int LayerStackModel::rms_seam(const NormW& nw, float* out, int T) {
+    const int W = info_.width;
+    const int st = ntk_rms_seam(out, W, x_, W, owed_.y, W, owed_.nb.w, residual_mult_, nw.w, T, W, eps_, stream_);
+    owed_.y = nullptr;
+    return st;
+}
+
+int LayerStackModel::scaled_layer(const Run& run, const StackLayer& L, int slot, int T, int pos0) {
+    LS_TRY(rms_seam(L.norm1, h1_, T));
+    if (L.mixer == kMixWindow) LS_TRY(run_window(L, run.cache + (size_t)slot * opt_.max_context * L.att.row(), T, pos0));
+    else if (L.mixer == kMixLatent) LS_TRY(run_mixer(L, run.cache + (size_t)slot * opt_.max_context * L.mix.row(), T, pos0, true));
+    else LS_TRY(run_gated_delta(L, run.state + (size_t)slot * L.gdl.state_floats(), T, pos0));
+    owed_ = Owed{mix_, L.norm1b};
+    if (!L.has_mlp) return NTK_OK;
+    LS_TRY(rms_seam(L.norm2, h2_, T));
+    LS_TRY(run_clipped_ff(L, T));
+    owed_ = Owed{ff_, L.norm2b};
+    return NTK_OK;
 }
 
 // gated linear attention: one product for [q | k | v | gate | a1 | residual gate], the decay's second projection, the recurrence (decay formed from its raw
@@ -983,7 +1163,8 @@ int LayerStackModel::norm_conv(const NormW& nw, const float* canon, float* conv_
 int LayerStackModel::settle(int T) {
     if (!owed_.y) return NTK_OK;
     const int W = info_.width;
-    const int st = ntk_layernorm(x_, W, owed_.y, W, owed_.nb.w, owed_.nb.b, T, W, eps_, 1, stream_);
+    const int st = form_.scaled ? ntk_rms_seam(nullptr, 0, x_, W, owed_.y, W, owed_.nb.w, residual_mult_, nullptr, T, W, eps_, stream_)
+                                : ntk_layernorm(x_, W, owed_.y, W, owed_.nb.w, owed_.nb.b, T, W, eps_, 1, stream_);
     owed_.y = nullptr;
     return st;
 }
@@ -1041,6 +1222,9 @@ int LayerStackModel::portion(int slot, const int* tokens_dev, int T, int pos0, c
         }
         if (form_.gated) {
             LS_TRY(gated_layer(r, L, slot, T, pos0));
+        } else if (form_.scaled) {
+            LS_TRY(scaled_layer(run, L, slot, T, pos0));
+            if (r + 1 == runs_.size() || (capture_ && capture_buf_)) LS_TRY(settle(T));
         } else if (form_.sequential) {
             LS_TRY(sequential_layer(run, L, slot, T, pos0));
             if (r + 1 == runs_.size() || (capture_ && capture_buf_)) LS_TRY(settle(T));
@@ -1059,9 +1243,10 @@ int LayerStackModel::portion(int slot, const int* tokens_dev, int T, int pos0, c
         d.N = info_.vocab; d.K = W;
         if (form_.gated) { LS_TRY(ntk_dyt(hn_, W, rows, W, final_norm_.w, final_norm_.b, final_norm_.alpha, n_want, W, stream_)); d.X = hn_; }
         else if (final_norm_.b) { LS_TRY(ntk_layernorm(hn_, W, rows, W, final_norm_.w, final_norm_.b, n_want, W, eps_, 0, stream_)); d.X = hn_; }
-        else if (n_want <= ntk_dense_few_rows()) { d.norm_w = final_norm_.w; d.norm_eps = eps_; d.norm_offset = 1.0f; }   // the output norm inside the head's launch
-        else { LS_TRY(ntk_rmsnorm_offset(hn_, final_norm_.w, nullptr, nullptr, W, rows, W, n_want, W, eps_, 1.0f, stream_)); d.X = hn_; }
+        else if (n_want <= ntk_dense_few_rows()) { d.norm_w = final_norm_.w; d.norm_eps = eps_; d.norm_offset = norm_offset_; }   // the output norm inside the head's launch
+        else { LS_TRY(ntk_rmsnorm_offset(hn_, final_norm_.w, nullptr, nullptr, W, rows, W, n_want, W, eps_, norm_offset_, stream_)); d.X = hn_; }
         LS_TRY(ntk_dense(&d, stream_));
+        if (logit_softcap_ > 0.0f) LS_TRY(ntk_softcap_rows(logits_out, info_.vocab, logit_softcap_, n_want, info_.vocab, stream_));
         if (logit_scale_ != 1.0f) LS_TRY(ntk_scale(logits_out, (long long)n_want * info_.vocab, logit_scale_, stream_));
     }
     return NTK_OK;

@@ -10,6 +10,9 @@
 //                result multiplied by sigmoid(W h + b) of the sublayer's input before it joins the stream, the stream that goes on after a layer a
 //                learned weighted sum of ALL layer results so far (and the embedding), a learned vector per position added to the embedding, scaled
 //                logits                                                                                                     -- "Tubazen"
+//   scaled       x += m * norm1b(mixer(norm1 x)), then x += m * norm2b(ff(norm2 x)): RMS norms with a plain weight before and after every sublayer, one
+//                fixed factor m on everything that joins the stream, scaled embedding, the embedding table as the head, capped logits
+//                                                                                                                           -- "Fifotar"
 //
 // Mechanisms are parsed into parameter structs and run by the operators of include/ntk_layers.h, so another family can list them in another order
 // or with other constants:
@@ -21,10 +24,15 @@
 //                 per head, silu gate (GlaMixer); "parallel": two mixers over the same input whose results are added with fixed weights -- grouped-query
 //                 softmax attention with projection biases, a query temperature growing with the position and a learned bias by bucketed distance
 //                 (BiasedAttention), beside a delta-rule recurrence with per-channel decay and removal rate (DeltaMixer);
+//                 in the scaled form "attention" is grouped-query attention without positions over CHUNKS of the sequence, with capped scores, a sink
+//                 in the softmax, values blended with those of the first such layer and an elementwise output gate (the same WindowMixer and kernels with
+//                 other parameters), "latent_attention" pairs rotated entries half against half and gates per head, and "delta" is the delta rule with
+//                 one decay and one write strength per head over unit queries and keys that went through a short convolution (GatedDeltaMixer);
 //   feed-forward  kind "moe": routed gated experts + an optional shared expert (MoeFeedForward: softmax or sigmoid scores, optional expert groups,
 //                 clipped or plain gated units); kind "dense": up, polynomial activation with unit-norm terms, down (DenseFeedForward), or in the
-//                 gated form a gated unit with the tanh form of gelu (GatedFeedForward).
-// What a sequence holds per layer run: cache rows per position (attention kinds), a recurrent state (lightning), the convolutions' last inputs.
+//                 gated form a gated unit with the tanh form of gelu (GatedFeedForward), in the scaled form the clipped gated unit of the experts as one
+//                 dense unit (GatedExperts with one member).
+// What a sequence holds per layer run: cache rows per position (attention kinds), a recurrent state (lightning, gla, delta rules), the convolutions' last inputs.
 #pragma once
 #include <string>
 #include <vector>
@@ -48,6 +56,8 @@ struct LatentMixer {
     float scale = 1.0f;
     int rot_dims = 0;
     float rot_mag = 1.0f;
+    int rot_layout = NTK_ROT_NEIGHBOURS;
+    bool head_gate = false;           // the output gate is one number per head (else one per head and value entry)
     double* rot_freq = nullptr;       // device [rot_dims / 2]
     DenseW in;                        // rows [query or query latent | kv_rank + rot_dim | gate] of one product over the normed input
     int q_off = 0, kv_off = 0, g_off = 0;
@@ -65,10 +75,29 @@ struct WindowMixer {                  // grouped-query attention, sliding window
     float diff = 0.0f, lambda = 0.0f; // maps == 2: out = (a_0 - lambda a_1) / rms * (1 - diff)
     int rot_dims = 0;
     double* rot_freq = nullptr;       // device [rot_dims / 2]
-    DenseW in;                        // rows [q | k | v] of one product over the mixer's input
-    int k_off = 0, v_off = 0;
+    int mask_mode = NTK_MASK_SLIDING; // what `window` means: a sliding window or chunks of the sequence
+    float softcap = 0.0f;             // > 0: scores pass cap * tanh(. / cap)
+    bool sink = false;                // one more exp(0) in every softmax's denominator
+    bool gated = false;               // elementwise sigmoid gate on the joined heads (its rows sit behind v in `in`)
+    bool v_mix = false, v_source = false;   // values blended with those of the first such layer (v_source: this IS that layer, it only keeps them)
+    float v_blend = 0.0f;
+    DenseW in;                        // rows [q | k | v (| gate)] of one product over the mixer's input
+    int k_off = 0, v_off = 0, g_off = 0;
     DenseW o;
     int row() const { return kv_heads * (maps * dim + vdim); }
+};
+
+struct GatedDeltaMixer {              // S' = w S, S = S' + k (beta (v - S'^T k))^T with one decay w = exp(-rate softplus(W_a h + bias)) and one beta = sigmoid(W_b h) per head
+    int heads = 0, kv_heads = 0, dim = 0, vdim = 0, taps = 1;
+    DenseW in;                        // rows [q | k | v | gate | beta | decay] of one product; q and k have kv_heads heads
+    int k_off = 0, v_off = 0, g_off = 0, b_off = 0, a_off = 0;
+    float* conv = nullptr;            // F32 [channels()][taps]: the short convolutions of q, k and v, one below the other
+    float *rates = nullptr, *dt_bias = nullptr;   // F32 [heads]: exp(A_log) and the bias inside the softplus
+    float* norm = nullptr;            // F32 [vdim], shared by the heads
+    DenseW o;
+    int channels() const { return 2 * kv_heads * dim + heads * vdim; }
+    size_t recurrent_floats() const { return (size_t)heads * dim * vdim; }
+    size_t state_floats() const { return recurrent_floats() + (size_t)(taps - 1) * channels(); }   // [S | the convolutions' last inputs]
 };
 
 struct LightningMixer {               // linear attention with a per-head decay; q, k, v through silu, gated RMS norm over the joined heads
@@ -153,8 +182,8 @@ struct DenseFeedForward {             // down(act(up h)), act = a N(z) + b N(z^2
 
 struct NormW { float* w = nullptr; float* b = nullptr; float alpha = 0.0f; };   // b: layer norm with bias (sequential form) / dynamic tanh with its alpha (gated form); none: RMS norm, weight around zero
 
-enum MixerKind { kMixLatent = 0, kMixWindow = 1, kMixLightning = 2, kMixGla = 3, kMixParallel = 4 };
-enum MlpKind { kMlpNone = 0, kMlpMoe = 1, kMlpDense = 2 };
+enum MixerKind { kMixLatent = 0, kMixWindow = 1, kMixLightning = 2, kMixGla = 3, kMixParallel = 4, kMixGatedDelta = 5 };
+enum MlpKind { kMlpNone = 0, kMlpMoe = 1, kMlpDense = 2, kMlpClipped = 3 };
 
 struct StackLayer {
     std::string type;
@@ -167,6 +196,8 @@ struct StackLayer {
     LightningMixer lin;
     GlaMixer gla;
     ParallelMixer par;
+    GatedDeltaMixer gdl;
+    GatedExperts cff;                       // scaled form: one dense clipped gated unit
     GatedFeedForward gff;
     float *rg1_b = nullptr, *rg2_b = nullptr;   // gated form: biases of the residual gates, F32 [width]
     float* depth = nullptr;                 // gated form: weights of the layer results so far (embedding first), device F32 [layer + 2]
@@ -175,13 +206,23 @@ struct StackLayer {
     MoeFeedForward mlp;
     DenseFeedForward ffn;
     int cache_row() const { return mixer == kMixLatent ? mix.row() : mixer == kMixWindow ? att.row() : mixer == kMixParallel ? par.left.row() : 0; }
-    size_t state_floats() const { return mixer == kMixLightning ? lin.state_floats() : mixer == kMixGla ? gla.state_floats() : mixer == kMixParallel ? par.right.state_floats() : 0; }
+    size_t state_floats() const {
+        return mixer == kMixLightning ? lin.state_floats() : mixer == kMixGla ? gla.state_floats() : mixer == kMixParallel ? par.right.state_floats() :
+               mixer == kMixGatedDelta ? gdl.state_floats() : 0;
+    }
 };
 
 // what a family fixes about its layers (everything else is read from config.json)
 struct StackForm {
     bool sequential = false;          // see the head of this file
-    bool gated = false;               // ... (neither: the parallel form)
+    bool gated = false;               // ...
+    bool scaled = false;              // ... (none of the three: the parallel form)
+    // the scaled form's mechanisms: what its design fixes about them
+    bool mask_chunks = false;         // an attention layer's mask.size is a chunk size (else a sliding window)
+    bool attention_sink = false;      // its softmax has a sink
+    bool attention_gate = false;      // ... and an elementwise output gate
+    bool rot_halves = false;          // rotated entries are paired half against half (else neighbours)
+    bool latent_head_gate = false;    // latent attention's output gate is one number per head
     bool loop_projection = true;      // the repeated span is entered through 'loop.in' over [stream ; embedding]
     int router_score = 0;             // 0 softmax, 1 sigmoid
     bool router_renorm = true;
@@ -225,6 +266,11 @@ private:
     int run_gla(const StackLayer& L, float* state, int T, int pos0);
     int run_parallel(const StackLayer& L, float* cache, float* state, int T, int pos0);
     int run_gated_ff(const StackLayer& L, int T);
+    int parse_gated_delta(const Json& L, GatedDeltaMixer& m);
+    int run_gated_delta(const StackLayer& L, float* state, int T, int pos0);
+    int run_clipped_ff(const StackLayer& L, int T);
+    int rms_seam(const NormW& nw, float* out, int T);
+    int scaled_layer(const Run& run, const StackLayer& L, int slot, int T, int pos0);
     int gated_layer(size_t r, const StackLayer& L, int slot, int T, int pos0);
     int parse_mlp(const Json& ml, const std::string& where, StackLayer& S);
     int upload_norm(const ModelFolder& f, const std::string& name, NormW& out);
@@ -236,12 +282,12 @@ private:
     int alloc_buffers();
     void* dev_alloc(size_t bytes);
     int portion(int slot, const int* tokens_dev, int T, int pos0, const int* want_dev, int n_want, float* logits_out);
-    int run_mixer(const StackLayer& L, float* cache, int T, int pos0);
+    int run_mixer(const StackLayer& L, float* cache, int T, int pos0, bool normed_input = false);
     int run_window(const StackLayer& L, float* cache, int T, int pos0);
     int run_lightning(const StackLayer& L, float* state, int T, int pos0);
     int run_moe(const StackLayer& L, int T, bool into_stream);
     int run_dense_ff(const StackLayer& L, int T);
-    int run_experts(const MoeFeedForward& M, const GatedExperts& ex, const float* h, float* gu, float* act, float* out, int rows, const int* offsets, const int* order, int top);
+    int run_experts(float glu_alpha, float glu_up_offset, const GatedExperts& ex, const float* h, float* gu, float* act, float* out, int rows, const int* offsets, const int* order, int top);
     int norm_conv(const NormW& nw, const float* canon, float* conv_state, float* out, int T, int pos0);
     int settle(int T);
     int sequential_layer(const Run& run, const StackLayer& L, int slot, int T, int pos0);
@@ -257,6 +303,8 @@ private:
     float eps_ = 1e-6f;
     int taps_ = 1;                    // the input convolutions' taps (sequential form)
     float embed_scale_ = 1.0f, logit_scale_ = 1.0f;
+    float residual_mult_ = 1.0f, logit_softcap_ = 0.0f;   // scaled form
+    float norm_offset_ = 1.0f;        // what is added to an RMS norm's stored weight: 1 where weights are stored around zero, 0 where plain
     bool has_state_ = false;          // some layer carries a recurrent state or convolution inputs: a slot can only be cut back to its start
     std::vector<StackLayer> layers_;
     std::vector<Run> runs_;
@@ -276,8 +324,8 @@ private:
     float *x_ = nullptr, *x0_ = nullptr, *cat_ = nullptr, *h1_ = nullptr, *h2_ = nullptr, *a_ = nullptr, *cq_ = nullptr, *q_ = nullptr, *qf_ = nullptr, *lat_ = nullptr,
           *att_ = nullptr, *kx_ = nullptr, *vx_ = nullptr, *mix_ = nullptr, *wts_ = nullptr, *sg_ = nullptr, *gu_ = nullptr, *act_ = nullptr, *dn_ = nullptr,
           *sgu_ = nullptr, *sact_ = nullptr, *sdn_ = nullptr, *scratch_ = nullptr, *xw_ = nullptr, *hn_ = nullptr, *hist_ = nullptr, *ff_ = nullptr, *zf_ = nullptr, *wscratch_ = nullptr, *lscratch_ = nullptr,
-          *results_ = nullptr, *zq_ = nullptr, *gu2_ = nullptr, *rscratch_ = nullptr;   // gated form: the layer results of the pass [runs + 1][chunk][width], decay pre-activations, [gate | up | residual gate]
-    int max_rec_ = 0, max_gu2_ = 0;
+          *results_ = nullptr, *zq_ = nullptr, *gu2_ = nullptr, *rscratch_ = nullptr, *cv_ = nullptr, *vfirst_ = nullptr;   // gated form: the layer results of the pass [runs + 1][chunk][width], decay pre-activations, [gate | up | residual gate]
+    int max_rec_ = 0, max_gu2_ = 0, max_conv_ = 0, max_gv_ = 0;   // (scaled form: convolution channels, key heads x value size of the blending attention layers)
     int *ids_ = nullptr, *offsets_ = nullptr, *order_ = nullptr, *where_ = nullptr, *tokens_dev_ = nullptr, *want_dev_ = nullptr;
     int* h_stage_ = nullptr;          // pinned: tokens and wanted places of the pass being launched
     float* logits_ = nullptr;

@@ -19,6 +19,10 @@
 // from segment to segment (recurrence_chain_kernel, a few small products in turn) and out_t += x(g)^T (P_t^T q_t) settles what every token's output was
 // still owed (recurrence_owed_kernel).  Only products of decays <= 1 appear, nothing is divided by a decay: no overflow whatever the decays are.
 // Within a segment the walk is the same whatever the portion; where the segments' borders fall changes the order of the sums, i.e. rounding only.
+//
+// The delta rule with one gate per head is the same walk with other vectors: S' = w S, S = S' - a u (u^T S') + a k v^T with a scalar w and a per head is
+// S = w S - (a u) ((w u)^T S) + k (a v)^T, so the pre-pass leaves (w u) where the walk takes the sum, (a u) where it removes, and a copy of the values
+// times a.  Unit queries and keys, q / k heads shared by several state heads and the per-head decay forms are the pre-pass's too.
 #include <algorithm>
 #include "common.hip.h"
 #include "../../include/ntk_layers.h"
@@ -43,6 +47,10 @@ struct RecArgs {
     float* pbuf;                     // [nseg][H][dn][dn]: the segment's whole transition
     float* lbuf;                     // [nseg][H][dn][dv]: the state the segment's own tokens leave (segment 0: from the sequence's state)
     float* sbuf;                     // [nseg][H][dn][dv]: the state at the segment's start
+    // the per-head options (pre-pass only)
+    int G, unit_q, unit_k, head_gates, write_gated;
+    const float* decay_rates;
+    float* vpacked;                  // [T][H][dv]: values times the removal rate (write_gated); the walk then reads these
 };
 
 constexpr int kRecFewTokens = 8;  // up to this many tokens (decoding) the walk forms its vectors itself: one launch
@@ -56,6 +64,7 @@ __device__ __forceinline__ float decay_of(float z, int form, float param) {
         return expf(-sp / param);
     }
     if (form == NTK_DECAY_EXP_SIGMOID) return expf(-param / (1.0f + expf(-z)));
+    if (form == NTK_DECAY_EXP_SOFTPLUS) return expf(-param * (fmaxf(z, 0.0f) + log1pf(expf(-fabsf(z)))));
     return z;
 }
 
@@ -66,23 +75,38 @@ __global__ __launch_bounds__(64) void gated_recurrence_prepare_kernel(const RecA
     const int lane = threadIdx.x, h = blockIdx.x % a.H;
     const long long t = blockIdx.x / a.H;
     float* dst = a.packed + (t * a.H + h) * NV * a.dn;
-    float ss = 0.0f;
+    const long long oq = (long long)(a.G > 0 ? h / (a.H / a.G) : h) * a.dn;      // where this state head's q and k lie
+    const long long oc = (long long)h * a.dn;                                     // ... and its per-channel gates
+    float ss = 0.0f, sq = 0.0f;
     for (int d = lane; d < a.dn; d += 64) {
-        const long long o = (long long)h * a.dn + d;
-        const float kk = a.k[t * a.ldk + o];
-        dst[d] = a.q[t * a.ldq + o] * a.q_scale;
-        dst[a.dn + d] = kk;
-        dst[2 * a.dn + d] = decay_of(a.wz[t * a.ldw + o] + (a.wb ? a.wb[o] : 0.0f), a.decay_form, a.decay_param);
+        const float kk = a.k[t * a.ldk + oq + d], qq = a.q[t * a.ldq + oq + d];
         ss = fmaf(kk, kk, ss);
+        sq = fmaf(qq, qq, sq);
+    }
+    const float inv_k = 1.0f / sqrtf(wave_sum(ss) + a.unit_eps);      // (the same sum in the same lane order as the staging of the walk forms it)
+    const float qmul = a.unit_q ? a.q_scale / sqrtf(wave_sum(sq) + a.unit_eps) : a.q_scale;
+    const float kmul = a.unit_k ? inv_k : 1.0f;
+    float wh = 1.0f, ah = 0.0f;                                        // one decay and one removal rate for the head
+    if (a.head_gates) {
+        wh = decay_of(a.wz[t * a.ldw + h] + (a.wb ? a.wb[h] : 0.0f), a.decay_form, a.decay_rates ? a.decay_rates[h] : a.decay_param);
+        if constexpr (DELTA) ah = 1.0f / (1.0f + expf(-(a.az[t * a.lda + h] + (a.ab ? a.ab[h] : 0.0f))));
+    }
+    for (int d = lane; d < a.dn; d += 64) {
+        const float kk = a.k[t * a.ldk + oq + d];
+        const float w = a.head_gates ? wh : decay_of(a.wz[t * a.ldw + oc + d] + (a.wb ? a.wb[oc + d] : 0.0f), a.decay_form, a.decay_rates ? a.decay_rates[h] : a.decay_param);
+        dst[d] = a.q[t * a.ldq + oq + d] * qmul;
+        dst[a.dn + d] = kk * kmul;
+        dst[2 * a.dn + d] = w;
+        if constexpr (DELTA) {
+            const float uu = kk * inv_k;
+            const float aa = a.head_gates ? ah : 1.0f / (1.0f + expf(-(a.az[t * a.lda + oc + d] + (a.ab ? a.ab[oc + d] : 0.0f))));
+            dst[3 * a.dn + d] = a.write_gated ? uu * w : uu;
+            dst[4 * a.dn + d] = uu * aa;
+        }
     }
     if constexpr (DELTA) {
-        const float inv = 1.0f / sqrtf(wave_sum(ss) + a.unit_eps);      // (the same sum in the same lane order as the staging of the walk forms it)
-        for (int d = lane; d < a.dn; d += 64) {
-            const long long o = (long long)h * a.dn + d;
-            const float uu = a.k[t * a.ldk + o] * inv;
-            dst[3 * a.dn + d] = uu;
-            dst[4 * a.dn + d] = uu * (1.0f / (1.0f + expf(-(a.az[t * a.lda + o] + (a.ab ? a.ab[o] : 0.0f)))));
-        }
+        if (a.write_gated)
+            for (int c = lane; c < a.dv; c += 64) a.vpacked[(t * a.H + h) * a.dv + c] = a.v[t * a.ldv + (long long)h * a.dv + c] * ah;
     }
 }
 
@@ -421,6 +445,7 @@ static int launch_rec_waves(const RecArgs& a0, hipStream_t s) {
         else hipLaunchKernelGGL(gated_recurrence_prepare_kernel<false>, dim3(a.T * a.H), dim3(64), 0, s, a);
         const int st = last_launch_status();
         if (st != NTK_OK) return st;
+        if (a.vpacked) { a.v = a.vpacked; a.ldv = a.H * a.dv; }
         if (delta) hipLaunchKernelGGL((gated_recurrence_kernel<SPLIT, RP, true, true, NW>), grid, dim3(NT), lds, s, a);
         else hipLaunchKernelGGL((gated_recurrence_kernel<SPLIT, RP, false, true, NW>), grid, dim3(NT), lds, s, a);
         if (a.nseg == 1) return last_launch_status();
@@ -473,30 +498,50 @@ static int rec_segments(int T, int H, int dn, int dv, bool removal) {
     return std::max(1, std::min(std::min(kRecMaxSegs, by_chip), T / kRecSegTokens));
 }
 
-size_t ntk_gated_recurrence_scratch(int T, int H, int dn, int dv, int removal) {
-    if (T <= kRecFewTokens) return 0;
-    size_t n = (size_t)T * H * (removal ? 5 : 3) * dn;
-    const int ns = rec_segments(T, H, dn, dv, removal != 0);
+// any of the per-head options: the vectors are always formed by the pre-pass
+static bool rec_needs_prepass(const ntk_gated_recurrence_desc* d) {
+    return d->G > 0 || d->unit_q || d->unit_k || d->head_gates || d->write_gated || d->decay_rates || d->decay_form == NTK_DECAY_EXP_SOFTPLUS;
+}
+
+static size_t rec_scratch(int T, int H, int dn, int dv, bool removal, bool always, bool values) {
+    if (T <= kRecFewTokens && !always) return 0;
+    size_t n = (size_t)T * H * (removal ? 5 : 3) * dn + (values ? (size_t)T * H * dv : 0);
+    const int ns = rec_segments(T, H, dn, dv, removal);
     if (ns > 1) n += (size_t)T * H * dn + (size_t)ns * H * dn * dn + 2 * (size_t)ns * H * dn * dv;
     return n;
+}
+
+size_t ntk_gated_recurrence_scratch(int T, int H, int dn, int dv, int removal) { return rec_scratch(T, H, dn, dv, removal != 0, false, false); }
+
+size_t ntk_gated_recurrence_scratch_ex(const ntk_gated_recurrence_desc* d) {
+    if (!d || d->T <= 0 || d->H <= 0 || d->dn <= 0 || d->dv <= 0) return 0;
+    return rec_scratch(d->T, d->H, d->dn, d->dv, d->az != nullptr, rec_needs_prepass(d), d->write_gated != 0);
 }
 
 int ntk_gated_recurrence(const ntk_gated_recurrence_desc* d, void* stream) {
     if (!d || !d->out || !d->q || !d->k || !d->v || !d->wz || !d->state) return NTK_E_NULL;
     if (d->T < 0 || d->H <= 0 || d->dn <= 0 || d->dv <= 0 || d->pos0 < 0 || d->dn > 1024) return NTK_E_SHAPE;
-    if (d->decay_form != NTK_DECAY_GIVEN && d->decay_form != NTK_DECAY_SIGMOID_ROOT && d->decay_form != NTK_DECAY_EXP_SIGMOID) return NTK_E_SHAPE;
+    if (d->decay_form != NTK_DECAY_GIVEN && d->decay_form != NTK_DECAY_SIGMOID_ROOT && d->decay_form != NTK_DECAY_EXP_SIGMOID && d->decay_form != NTK_DECAY_EXP_SOFTPLUS)
+        return NTK_E_SHAPE;
     if (d->decay_form == NTK_DECAY_SIGMOID_ROOT && !(d->decay_param > 0.0f)) return NTK_E_SHAPE;
-    const int hd = d->H * d->dn;
-    if (d->ldq < hd || d->ldk < hd || d->ldw < hd || (d->az && d->lda < hd) || d->ldv < d->H * d->dv || d->ldo < d->H * d->dv) return NTK_E_SHAPE;
+    if (d->G < 0 || (d->G > 0 && d->H % d->G)) return NTK_E_SHAPE;
+    if (d->write_gated && (!d->az || !d->head_gates)) return NTK_E_SHAPE;   // (the write is scaled by ONE rate per head)
+    const int hd = d->H * d->dn, qd = (d->G > 0 ? d->G : d->H) * d->dn, gd = d->head_gates ? d->H : hd;
+    if (d->ldq < qd || d->ldk < qd || d->ldw < gd || (d->az && d->lda < gd) || d->ldv < d->H * d->dv || d->ldo < d->H * d->dv) return NTK_E_SHAPE;
     if (d->T == 0) return NTK_OK;
+    const bool always = rec_needs_prepass(d);
+    if (always && !d->scratch) return NTK_E_NULL;
     RecArgs a{d->out, d->ldo, d->q, d->ldq, d->k, d->ldk, d->v, d->ldv, d->wz, d->ldw, d->wb, d->decay_form, d->decay_param, d->az, d->lda, d->ab, d->unit_eps,
-              d->state, d->H, d->dn, d->dv, d->q_scale, d->pos0, d->T, 0, d->T > kRecFewTokens ? d->scratch : nullptr, 1, d->T, nullptr, nullptr, nullptr, nullptr};
+              d->state, d->H, d->dn, d->dv, d->q_scale, d->pos0, d->T, 0, (d->T > kRecFewTokens || always) ? d->scratch : nullptr, 1, d->T, nullptr, nullptr, nullptr, nullptr,
+              d->G, d->unit_q, d->unit_k, d->head_gates, d->write_gated, d->decay_rates, nullptr};
     if (a.packed) {
+        float* next = a.packed + (size_t)d->T * d->H * (d->az ? 5 : 3) * d->dn;
+        if (d->write_gated) { a.vpacked = next; next += (size_t)d->T * d->H * d->dv; }
         a.nseg = rec_segments(d->T, d->H, d->dn, d->dv, d->az != nullptr);
         if (a.nseg > 1) {
             a.seg_len = (d->T + a.nseg - 1) / a.nseg;
             a.nseg = (d->T + a.seg_len - 1) / a.seg_len;
-            a.rbuf = a.packed + (size_t)d->T * d->H * (d->az ? 5 : 3) * d->dn;
+            a.rbuf = next;
             a.pbuf = a.rbuf + (size_t)d->T * d->H * d->dn;
             a.lbuf = a.pbuf + (size_t)a.nseg * d->H * d->dn * d->dn;
             a.sbuf = a.lbuf + (size_t)a.nseg * d->H * d->dn * d->dv;

@@ -18,7 +18,7 @@ namespace ntk {
 // one workgroup per token: latent / rms * w and the rotated key part into the cache row, the rotated part of every query head in place.
 // Angles in double (position times frequency, then cos / sin), applied in F32.
 __global__ __launch_bounds__(256) void latent_prepare_kernel(float* cache, int row, const float* kv, int ldkv, const float* norm_w, float eps, int R, int dr,
-                                                             float* q, int ldq, int H, int qd, const double* freq, float mag, int dims, int pos0) {
+                                                             float* q, int ldq, int H, int qd, const double* freq, float mag, int dims, int pos0, int halves) {
     __shared__ float red[16];
     extern __shared__ float cs[];   // [dims / 2] cos, [dims / 2] sin
     const int t = blockIdx.x, pos = pos0 + t;
@@ -35,22 +35,23 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(float* cache, int r
     ss = block_sum(ss, red);   // (its barriers also publish cs)
     const float inv = 1.0f / sqrtf(ss / (float)R + eps);
     for (int i = threadIdx.x; i < R; i += 256) dst[i] = src[i] * inv * norm_w[i];
+    const int pair = halves ? half : 1, step = halves ? 1 : 2;   // pair i = entries (i * step, i * step + pair)
     for (int i = threadIdx.x; i < half; i += 256) {
         float ra, rb;
-        rope_rotate(src[R + 2 * i], src[R + 2 * i + 1], cs[i], cs[half + i], ra, rb);
-        dst[R + 2 * i] = ra;
-        dst[R + 2 * i + 1] = rb;
+        rope_rotate(src[R + step * i], src[R + step * i + pair], cs[i], cs[half + i], ra, rb);
+        dst[R + step * i] = ra;
+        dst[R + step * i + pair] = rb;
     }
     for (int i = dims + threadIdx.x; i < dr; i += 256) dst[R + i] = src[R + i];
     if (q) {
         float* qt = q + (long long)t * ldq;
         for (int j = threadIdx.x; j < H * half; j += 256) {
             const int h = j / half, i = j % half;
-            float* p = qt + h * qd + (qd - dr) + 2 * i;
+            float* p = qt + h * qd + (qd - dr) + step * i;
             float ra, rb;
-            rope_rotate(p[0], p[1], cs[i], cs[half + i], ra, rb);
+            rope_rotate(p[0], p[pair], cs[i], cs[half + i], ra, rb);
             p[0] = ra;
-            p[1] = rb;
+            p[pair] = rb;
         }
     }
 }
@@ -422,7 +423,7 @@ __global__ __launch_bounds__(256) void latent_fold_query_kernel(float* qf, const
 // out[t][h * dv + v] = W_uv[h * dv + v][:] . lat[t][h][:] (* sigmoid(gate));  grid (dv / 16, H, T): a wave owns 4 outputs and walks their rows together
 template <typename WT>
 __global__ __launch_bounds__(256) void latent_unfold_value_kernel(float* out, int ldo, const float* lat, const WT* w, const float* gate, int ldg, int H, int dv,
-                                                                 int R) {
+                                                                 int R, int head_gate) {
     extern __shared__ float ls[];
     const int h = blockIdx.y, t = blockIdx.z;
     const float* lh = lat + ((long long)t * H + h) * R;
@@ -449,7 +450,7 @@ __global__ __launch_bounds__(256) void latent_unfold_value_kernel(float* out, in
     for (int i = 0; i < 4; ++i) {
         float tsum = wave_sum_lane63(s[i]);
         if (lane == 63 && v0 + i < dv) {
-            if (gate) tsum *= 1.0f / (1.0f + expf(-gate[(long long)t * ldg + h * dv + v0 + i]));
+            if (gate) tsum *= 1.0f / (1.0f + expf(-gate[(long long)t * ldg + (head_gate ? h : h * dv + v0 + i)]));
             out[(long long)t * ldo + h * dv + v0 + i] = tsum;
         }
     }
@@ -469,9 +470,10 @@ int ntk_latent_prepare(float* cache, int row, const float* kv, int ldkv, const f
     if (!cache || !kv || !norm_w || !rot || !rot->freq) return NTK_E_NULL;
     if (T < 0 || kv_rank <= 0 || rot_dim < 0 || rot->dims < 0 || (rot->dims & 1) || rot->dims > rot_dim || row < kv_rank + rot_dim || ldkv < kv_rank + rot_dim || pos0 < 0) return NTK_E_SHAPE;
     if (q && (H <= 0 || qd < rot_dim || ldq < H * qd)) return NTK_E_SHAPE;
+    if (rot->layout != NTK_ROT_NEIGHBOURS && rot->layout != NTK_ROT_HALVES) return NTK_E_SHAPE;
     if (T == 0) return NTK_OK;
     hipLaunchKernelGGL(latent_prepare_kernel, dim3(T), dim3(256), (size_t)(rot_dim + 2) * sizeof(float), resolve_stream(stream), cache, row, kv, ldkv, norm_w,
-                       eps, kv_rank, rot_dim, q, ldq, H, qd, rot->freq, rot->mag, rot->dims, pos0);
+                       eps, kv_rank, rot_dim, q, ldq, H, qd, rot->freq, rot->mag, rot->dims, pos0, rot->layout == NTK_ROT_HALVES ? 1 : 0);
     return last_launch_status();
 }
 
@@ -542,13 +544,18 @@ int ntk_latent_fold_query(float* qf, const float* q, int ldq, const void* w_uk, 
 
 int ntk_latent_unfold_value(float* out, int ldo, const float* lat, const void* w_uv, int wdtype, const float* gate, int ldg, int T, int H, int dv, int R,
                             void* stream) {
+    return ntk_latent_unfold_value_ex(out, ldo, lat, w_uv, wdtype, gate, ldg, 0, T, H, dv, R, stream);
+}
+
+int ntk_latent_unfold_value_ex(float* out, int ldo, const float* lat, const void* w_uv, int wdtype, const float* gate, int ldg, int head_gate, int T, int H, int dv,
+                               int R, void* stream) {
     if (!out || !lat || !w_uv) return NTK_E_NULL;
     if (T < 0 || H <= 0 || dv <= 0 || R <= 0) return NTK_E_SHAPE;
     if (T == 0) return NTK_OK;
     const size_t lds = (size_t)R * sizeof(float);
     const dim3 grid((dv + 15) / 16, H, T);
-    if (wdtype == NTK_DT_BF16) hipLaunchKernelGGL(latent_unfold_value_kernel<uint16_t>, grid, dim3(256), lds, resolve_stream(stream), out, ldo, lat, (const uint16_t*)w_uv, gate, ldg, H, dv, R);
-    else if (wdtype == NTK_DT_F32) hipLaunchKernelGGL(latent_unfold_value_kernel<float>, grid, dim3(256), lds, resolve_stream(stream), out, ldo, lat, (const float*)w_uv, gate, ldg, H, dv, R);
+    if (wdtype == NTK_DT_BF16) hipLaunchKernelGGL(latent_unfold_value_kernel<uint16_t>, grid, dim3(256), lds, resolve_stream(stream), out, ldo, lat, (const uint16_t*)w_uv, gate, ldg, H, dv, R, head_gate);
+    else if (wdtype == NTK_DT_F32) hipLaunchKernelGGL(latent_unfold_value_kernel<float>, grid, dim3(256), lds, resolve_stream(stream), out, ldo, lat, (const float*)w_uv, gate, ldg, H, dv, R, head_gate);
     else return NTK_E_DTYPE;
     return last_launch_status();
 }

@@ -488,3 +488,153 @@ int ntk_gated_seam(const ntk_gated_seam_desc* d, void* stream) {
     hipLaunchKernelGGL(ntk::gated_seam_kernel, dim3((d->n + 255) / 256, d->T), dim3(256), 0, resolve_stream(stream), a);
     return last_launch_status();
 }
+
+// ---------------------------------------------------------------------------------------------------------------- layers with scaled, RMS-normed sublayer results
+// The seam between two sublayers: the result the stream is still owed joins it (RMS norm, weight, a fixed factor), and the norm in front of the next sublayer
+// reads the row the same launch has just written (a thread reads back only what it wrote itself).  The short convolution of a recurrent mixer's projections
+// carries its last inputs from portion to portion; one token is one launch (a channel's history belongs to the thread that owns the channel).
+namespace ntk {
+
+template <int NT>
+__global__ __launch_bounds__(NT) void rms_seam_kernel(float* h, int ldh, float* x, int ldx, const float* add_y, int ldy, const float* add_w, float mult, const float* w,
+                                                      int n, float eps) {
+    __shared__ float red[16];
+    constexpr int KEEP = 4096 / NT;              // a thread's first entries stay in registers: rows up to 4096 wide cross memory once
+    float* xr = x + (long long)blockIdx.x * ldx;
+    float v[KEEP];
+    if (add_y) {
+        const float* yr = add_y + (long long)blockIdx.x * ldy;
+        float ss = 0.0f;
+#pragma unroll
+        for (int k = 0; k < KEEP; ++k) {
+            const int i = threadIdx.x + NT * k;
+            v[k] = i < n ? yr[i] : 0.0f;
+            ss = fmaf(v[k], v[k], ss);
+        }
+        for (int i = threadIdx.x + NT * KEEP; i < n; i += NT) ss = fmaf(yr[i], yr[i], ss);
+        const float inv = mult / sqrtf(block_sum(ss, red) / (float)n + eps);
+#pragma unroll
+        for (int k = 0; k < KEEP; ++k) {
+            const int i = threadIdx.x + NT * k;
+            if (i < n) { v[k] = fmaf(v[k] * inv, add_w[i], xr[i]); xr[i] = v[k]; }
+        }
+        for (int i = threadIdx.x + NT * KEEP; i < n; i += NT) xr[i] = fmaf(yr[i] * inv, add_w[i], xr[i]);
+    } else {
+#pragma unroll
+        for (int k = 0; k < KEEP; ++k) {
+            const int i = threadIdx.x + NT * k;
+            v[k] = i < n ? xr[i] : 0.0f;
+        }
+    }
+    if (!h) return;                              // (uniform over the launch)
+    float ss = 0.0f;
+#pragma unroll
+    for (int k = 0; k < KEEP; ++k)
+        if ((int)threadIdx.x + NT * k < n) ss = fmaf(v[k], v[k], ss);
+    for (int i = threadIdx.x + NT * KEEP; i < n; i += NT) ss = fmaf(xr[i], xr[i], ss);
+    const float inv = 1.0f / sqrtf(block_sum(ss, red) / (float)n + eps);
+    float* hr = h + (long long)blockIdx.x * ldh;
+#pragma unroll
+    for (int k = 0; k < KEEP; ++k) {
+        const int i = threadIdx.x + NT * k;
+        if (i < n) hr[i] = v[k] * inv * w[i];
+    }
+    for (int i = threadIdx.x + NT * KEEP; i < n; i += NT) hr[i] = xr[i] * inv * w[i];
+}
+
+constexpr int kConvMaxTaps = 16;
+__device__ __forceinline__ float conv_act(float s, int act) { return act == 1 ? s / (1.0f + expf(-s)) : s; }
+
+// the input `back` rows before row t of the portion: the portion's own row, a carried one, or zero before the sequence's start
+__device__ __forceinline__ float conv_input(const float* x, int ldx, const float* state, int taps, int pos0, int n, int c, int idx) {
+    if (idx >= 0) return x[(long long)idx * ldx + c];
+    if (pos0 + idx < 0) return 0.0f;
+    return state[(long long)(taps - 1 + idx) * n + c];   // carried row taps - 1 + idx: the row that lay idx before this portion
+}
+
+// blocks y < T: the outputs; one more launch shifts the carried rows (they are read here)
+__global__ void causal_conv_act_kernel(float* y, int ldy, const float* x, int ldx, const float* w, const float* state, int taps, int act, int pos0, int n) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x, t = blockIdx.y;
+    if (c >= n) return;
+    float s = 0.0f;
+    for (int j = 0; j < taps; ++j) s = fmaf(w[(long long)c * taps + j], conv_input(x, ldx, state, taps, pos0, n, c, t - (taps - 1) + j), s);
+    y[(long long)t * ldy + c] = conv_act(s, act);
+}
+
+// the carried rows after the portion: a thread owns a channel, reads its taps - 1 new rows (some of them old carried rows when the portion is shorter) and
+// then writes them.  T == 1 with an output: the whole operator for one token in this one launch.
+__global__ void causal_conv_carry_kernel(float* y, const float* x, int ldx, const float* w, float* state, int taps, int act, int pos0, int T, int n) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= n) return;
+    float keep[kConvMaxTaps];
+#pragma unroll
+    for (int r = 0; r < kConvMaxTaps; ++r)
+        if (r < taps) keep[r] = conv_input(x, ldx, state, taps, pos0, n, c, T - taps + r);      // rows T - taps .. T - 1 (the first only for the output)
+    if (y) {
+        float s = 0.0f;
+#pragma unroll
+        for (int r = 0; r < kConvMaxTaps; ++r)
+            if (r < taps) s = fmaf(w[(long long)c * taps + r], keep[r], s);
+        y[c] = conv_act(s, act);
+    }
+#pragma unroll
+    for (int r = 1; r < kConvMaxTaps; ++r)
+        if (r < taps) state[(long long)(r - 1) * n + c] = keep[r];
+}
+
+__global__ void softcap_rows_kernel(float* x, int ldx, float cap, int n) {
+    const long long t = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[t * ldx + i] = cap * tanhf(x[t * ldx + i] / cap);
+}
+
+__global__ void head_gate_kernel(float* y, int ldy, const float* g, int ldg, int H, int dv) {
+    const long long t = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= H * dv) return;
+    y[t * ldy + i] *= sigmoidf_(g[t * ldg + i / dv]);
+}
+
+}  // namespace ntk
+
+int ntk_rms_seam(float* h, int ldh, float* x, int ldx, const float* add_y, int ldy, const float* add_w, float mult, const float* w, int T, int n, float eps,
+                 void* stream) {
+    if (!x || (add_y && !add_w) || (h && !w)) return NTK_E_NULL;
+    if (T < 0 || n <= 0 || ldx < n || (h && ldh < n) || (add_y && ldy < n)) return NTK_E_SHAPE;
+    if (T == 0 || (!add_y && !h)) return NTK_OK;
+    if (T <= kFewRows) hipLaunchKernelGGL(ntk::rms_seam_kernel<1024>, dim3(T), dim3(1024), 0, resolve_stream(stream), h, ldh, x, ldx, add_y, ldy, add_w, mult, w, n, eps);
+    else hipLaunchKernelGGL(ntk::rms_seam_kernel<256>, dim3(T), dim3(256), 0, resolve_stream(stream), h, ldh, x, ldx, add_y, ldy, add_w, mult, w, n, eps);
+    return last_launch_status();
+}
+
+int ntk_causal_conv_act(float* y, int ldy, const float* x, int ldx, const float* w, float* state, int taps, int act, int pos0, int T, int n, void* stream) {
+    if (!y || !x || !w || (taps > 1 && !state)) return NTK_E_NULL;
+    if (T < 0 || n <= 0 || ldy < n || ldx < n || taps < 1 || taps > ntk::kConvMaxTaps || pos0 < 0 || act < 0 || act > 1) return NTK_E_SHAPE;
+    if (T == 0) return NTK_OK;
+    hipStream_t s = resolve_stream(stream);
+    if (T == 1) {
+        hipLaunchKernelGGL(ntk::causal_conv_carry_kernel, dim3((n + 255) / 256), dim3(256), 0, s, y, x, ldx, w, state, taps, act, pos0, T, n);
+        return last_launch_status();
+    }
+    hipLaunchKernelGGL(ntk::causal_conv_act_kernel, dim3((n + 255) / 256, T), dim3(256), 0, s, y, ldy, x, ldx, w, (const float*)state, taps, act, pos0, n);
+    const int st = last_launch_status();
+    if (st != NTK_OK || taps == 1) return st;
+    hipLaunchKernelGGL(ntk::causal_conv_carry_kernel, dim3((n + 255) / 256), dim3(256), 0, s, (float*)nullptr, x, ldx, w, state, taps, act, pos0, T, n);
+    return last_launch_status();
+}
+
+int ntk_softcap_rows(float* x, int ldx, float cap, int T, int n, void* stream) {
+    if (!x) return NTK_E_NULL;
+    if (T < 0 || n <= 0 || ldx < n || !(cap > 0.0f)) return NTK_E_SHAPE;
+    if (T == 0) return NTK_OK;
+    hipLaunchKernelGGL(ntk::softcap_rows_kernel, dim3((n + 255) / 256, T), dim3(256), 0, resolve_stream(stream), x, ldx, cap, n);
+    return last_launch_status();
+}
+
+int ntk_head_gate(float* y, int ldy, const float* g, int ldg, int T, int H, int dv, void* stream) {
+    if (!y || !g) return NTK_E_NULL;
+    if (T < 0 || H <= 0 || dv <= 0 || ldy < H * dv || ldg < H) return NTK_E_SHAPE;
+    if (T == 0) return NTK_OK;
+    hipLaunchKernelGGL(ntk::head_gate_kernel, dim3((H * dv + 255) / 256, T), dim3(256), 0, resolve_stream(stream), y, ldy, g, ldg, H, dv);
+    return last_launch_status();
+}

@@ -1,6 +1,8 @@
 // window_attention.hip -- grouped-query softmax attention over a cache of rotated keys and values: causal, optional sliding window, one or two score
 // maps per head over the same values (two maps: the differential pair out = a_0 - lambda * a_1), optional unit norm of every head's output, optional
-// learned bias by bucketed distance on the scaled score (a table of distances -> buckets, a table of buckets x heads).
+// learned bias by bucketed distance on the scaled score (a table of distances -> buckets, a table of buckets x heads), optional cap on the score
+// (cap * tanh(score / cap)), optional sink (a key of score 0 without a value in every softmax), and instead of the sliding window a mask of chunks
+// (a query sees the keys of its own chunk of `window` positions, counted from position 0, up to itself).
 //
 // Cache row of a position: [G][maps][dn] rotated keys | [G][dv] values, F32.  Scores, softmax, weights and sums are F32 on the vector units.
 // A workgroup owns 16 (token, head) rows of ONE key/value head -- consecutive tokens times the heads that share it, so a key or value slab that was
@@ -17,7 +19,8 @@ namespace ntk {
 // Optional: what the projections left to their consumer -- bias vectors on q, k and v, and a query temperature that grows with the position.
 __global__ __launch_bounds__(256) void window_prepare_kernel(float* cache, int row, float* q, int ldq, const float* k, int ldk, const float* v, int ldv, int nq, int nk,
                                                              int dn, int nv, const double* freq, float mag, int dims, int pos0, const float* qb, const float* kb,
-                                                             const float* vb, float temp_coef, double temp_every) {
+                                                             const float* vb, float temp_coef, double temp_every, int halves, const float* v_other, int ld_other,
+                                                             float v_blend, float* v_keep, int ld_keep) {
     extern __shared__ float cs[];   // [dims / 2] cos, [dims / 2] sin
     const int t = blockIdx.x, pos = pos0 + t;
     const int half = dims / 2;
@@ -37,26 +40,32 @@ __global__ __launch_bounds__(256) void window_prepare_kernel(float* cache, int r
     float* qt = q + (long long)t * ldq;
     const float* kt = k + (long long)t * ldk;
     const float* vt = v + (long long)t * ldv;
+    const int pair = halves ? half : 1, step = halves ? 1 : 2;   // pair i = entries (i * step, i * step + pair)
     for (int j = threadIdx.x; j < nq * half; j += 256) {       // nq = heads x maps vectors of dn
-        float* p = qt + (j / half) * dn + 2 * (j % half);
+        float* p = qt + (j / half) * dn + step * (j % half);
         float ra, rb;
-        rope_rotate(p[0], p[1], cs[j % half], cs[half + j % half], ra, rb);
+        rope_rotate(p[0], p[pair], cs[j % half], cs[half + j % half], ra, rb);
         p[0] = ra;
-        p[1] = rb;
+        p[pair] = rb;
     }
     for (int j = threadIdx.x; j < nk * half; j += 256) {
-        const int o = (j / half) * dn + 2 * (j % half);
+        const int o = (j / half) * dn + step * (j % half);
         float ra, rb;
-        rope_rotate(kt[o] + (kb ? kb[o] : 0.0f), kt[o + 1] + (kb ? kb[o + 1] : 0.0f), cs[j % half], cs[half + j % half], ra, rb);
+        rope_rotate(kt[o] + (kb ? kb[o] : 0.0f), kt[o + pair] + (kb ? kb[o + pair] : 0.0f), cs[j % half], cs[half + j % half], ra, rb);
         dst[o] = ra;
-        dst[o + 1] = rb;
+        dst[o + pair] = rb;
     }
     const int rest = dn - dims;
     for (int j = threadIdx.x; j < nk * rest; j += 256) {
         const int o = (j / rest) * dn + dims + j % rest;
         dst[o] = kt[o] + (kb ? kb[o] : 0.0f);
     }
-    for (int j = threadIdx.x; j < nv; j += 256) dst[nk * dn + j] = vt[j] + (vb ? vb[j] : 0.0f);
+    for (int j = threadIdx.x; j < nv; j += 256) {
+        float vv = vt[j] + (vb ? vb[j] : 0.0f);
+        if (v_keep) v_keep[(long long)t * ld_keep + j] = vv;
+        if (v_other) vv = fmaf(v_blend, v_other[(long long)t * ld_other + j], (1.0f - v_blend) * vv);
+        dst[nk * dn + j] = vv;
+    }
 }
 
 struct WinArgs {
@@ -68,7 +77,14 @@ struct WinArgs {
     int sub_norm; float eps, out_scale;
     int splits; float* scratch;       // splits > 1: states [T * H][splits][maps][2 + dv]
     const float* rel; const int* bucket_of; int n_dist;   // rel != NULL: rel[bucket_of[min(distance, n_dist - 1)] * H + head] joins the scaled score
+    int chunks; float softcap; int sink;                  // chunks != 0: `window` is a chunk size
 };
+
+// first key a query at position p sees
+__device__ __forceinline__ int first_visible(int p, int window, int chunks) {
+    if (window <= 0) return 0;
+    return chunks ? (p / window) * window : max(0, p - window + 1);
+}
 
 constexpr int WROWS = 16, WQPW = 4, WKCH = 64, WSLAB = 64, WMAXC = 8;   // dv <= WMAXC * WSLAB
 
@@ -104,7 +120,7 @@ __global__ __launch_bounds__(256) void window_attention_kernel(const WinArgs a) 
     const int row0 = blockIdx.x * WROWS;
     const int last = min(row0 + WROWS, n_rows) - 1;
     const int pmin = a.pos0 + row0 / R, pmax = a.pos0 + last / R;
-    const int jlo = a.window > 0 ? max(0, pmin - a.window + 1) : 0;
+    const int jlo = first_visible(pmin, a.window, a.chunks);
     const int jhi = pmax;   // inclusive
     // queries into LDS
     for (int e0 = threadIdx.x; e0 < WROWS * M * DNP; e0 += 256 * 4) {     // (four of a thread's entries asked for before the first is stored)
@@ -126,9 +142,11 @@ __global__ __launch_bounds__(256) void window_attention_kernel(const WinArgs a) 
         const int rho = row0 + wave * WQPW + i;
         rpos[i] = rho < n_rows ? a.pos0 + rho / R : -1;
         rhead[i] = g * R + rho % R;
+        // the sink is a key of score 0 without a value: the running maximum and sum start from it (in the first part only when the keys are split)
+        const bool sunk = a.sink && (a.splits <= 1 || blockIdx.z == 0);
 #pragma unroll
         for (int m = 0; m < M; ++m) {
-            mx[m][i] = -INFINITY; l[m][i] = 0.0f;
+            mx[m][i] = sunk ? 0.0f : -INFINITY; l[m][i] = sunk ? 1.0f : 0.0f;
 #pragma unroll
             for (int c = 0; c < WMAXC; ++c) acc[m][i][c] = 0.0f;
         }
@@ -173,9 +191,10 @@ __global__ __launch_bounds__(256) void window_attention_kernel(const WinArgs a) 
             // ---- online softmax of map m, weights to LDS
 #pragma unroll
             for (int i = 0; i < WQPW; ++i) {
-                const bool vis = lane < nk && rpos[i] >= 0 && j <= rpos[i] && (a.window <= 0 || rpos[i] - j < a.window);
+                const bool vis = lane < nk && rpos[i] >= 0 && j <= rpos[i] && j >= first_visible(rpos[i], a.window, a.chunks);
                 float sv = vis ? s[i] * a.scale : -INFINITY;
                 if (a.rel && vis) sv += a.rel[(long long)a.bucket_of[min(rpos[i] - j, a.n_dist - 1)] * a.H + rhead[i]];
+                if (a.softcap > 0.0f && vis) sv = a.softcap * tanhf(sv / a.softcap);
                 const float mn = fmaxf(mx[m][i], wave_max(sv));
                 const float ms = mn == -INFINITY ? 0.0f : mn;
                 const float p = vis ? expf(sv - ms) : 0.0f;
@@ -297,8 +316,9 @@ static int window_splits(int T, int H, int G, int nkeys) {
     if (s > 64) s = 64;
     return s < 2 ? 1 : s;
 }
-static int window_keys(int pos0, int T, int window) {
+static int window_keys(int pos0, int T, int window, int chunks) {
     const int all = pos0 + T;
+    if (chunks && window > 0) return all - (pos0 / window) * window;     // from the start of the first token's chunk
     return window > 0 && window + T - 1 < all ? window + T - 1 : all;
 }
 
@@ -314,14 +334,24 @@ int ntk_window_prepare(float* cache, int row, float* q, int ldq, const float* k,
 int ntk_window_prepare_biased(float* cache, int row, float* q, int ldq, const float* k, int ldk, const float* v, int ldv, int H, int G, int maps, int dn, int dv,
                               const ntk_rotary* rot, const float* qb, const float* kb, const float* vb, float temp_coef, double temp_every, int pos0, int T,
                               void* stream) {
-    if (!cache || !q || !k || !v || !rot || (rot->dims > 0 && !rot->freq)) return NTK_E_NULL;
-    if (temp_coef != 0.0f && !(temp_every > 0.0)) return NTK_E_SHAPE;
-    if (T < 0 || H <= 0 || G <= 0 || H % G || maps < 1 || dn <= 0 || dv <= 0 || pos0 < 0) return NTK_E_SHAPE;
-    if (rot->dims < 0 || (rot->dims & 1) || rot->dims > dn) return NTK_E_SHAPE;
-    if (row < G * (maps * dn + dv) || ldq < H * maps * dn || ldk < G * maps * dn || ldv < G * dv) return NTK_E_SHAPE;
-    if (T == 0) return NTK_OK;
-    hipLaunchKernelGGL(window_prepare_kernel, dim3(T), dim3(256), (size_t)(rot->dims + 2) * sizeof(float), resolve_stream(stream), cache, row, q, ldq, k, ldk, v, ldv,
-                       H * maps, G * maps, dn, G * dv, rot->freq, rot->mag, rot->dims, pos0, qb, kb, vb, temp_coef, temp_every);
+    ntk_window_prepare_desc d{};
+    d.cache = cache; d.row = row; d.q = q; d.ldq = ldq; d.k = k; d.ldk = ldk; d.v = v; d.ldv = ldv; d.H = H; d.G = G; d.maps = maps; d.dn = dn; d.dv = dv; d.rot = rot;
+    d.qb = qb; d.kb = kb; d.vb = vb; d.temp_coef = temp_coef; d.temp_every = temp_every; d.pos0 = pos0; d.T = T;
+    return ntk_window_prepare_ex(&d, stream);
+}
+
+int ntk_window_prepare_ex(const ntk_window_prepare_desc* d, void* stream) {
+    if (!d || !d->cache || !d->q || !d->k || !d->v || !d->rot || (d->rot->dims > 0 && !d->rot->freq)) return NTK_E_NULL;
+    const ntk_rotary* rot = d->rot;
+    if (d->temp_coef != 0.0f && !(d->temp_every > 0.0)) return NTK_E_SHAPE;
+    if (d->T < 0 || d->H <= 0 || d->G <= 0 || d->H % d->G || d->maps < 1 || d->dn <= 0 || d->dv <= 0 || d->pos0 < 0) return NTK_E_SHAPE;
+    if (rot->dims < 0 || (rot->dims & 1) || rot->dims > d->dn || (rot->layout != NTK_ROT_NEIGHBOURS && rot->layout != NTK_ROT_HALVES)) return NTK_E_SHAPE;
+    if (d->row < d->G * (d->maps * d->dn + d->dv) || d->ldq < d->H * d->maps * d->dn || d->ldk < d->G * d->maps * d->dn || d->ldv < d->G * d->dv) return NTK_E_SHAPE;
+    if ((d->v_other && d->ld_other < d->G * d->dv) || (d->v_keep && d->ld_keep < d->G * d->dv)) return NTK_E_SHAPE;
+    if (d->T == 0) return NTK_OK;
+    hipLaunchKernelGGL(window_prepare_kernel, dim3(d->T), dim3(256), (size_t)(rot->dims + 2) * sizeof(float), resolve_stream(stream), d->cache, d->row, d->q, d->ldq,
+                       d->k, d->ldk, d->v, d->ldv, d->H * d->maps, d->G * d->maps, d->dn, d->G * d->dv, rot->freq, rot->mag, rot->dims, d->pos0, d->qb, d->kb, d->vb,
+                       d->temp_coef, d->temp_every, rot->layout == NTK_ROT_HALVES ? 1 : 0, d->v_other, d->ld_other, d->v_blend, d->v_keep, d->ld_keep);
     return last_launch_status();
 }
 
@@ -341,7 +371,9 @@ int ntk_window_attention(const ntk_window_attention_desc* d, void* stream) {
     WinArgs a{};
     a.out = d->out; a.ldo = d->ldo; a.q = d->q; a.ldq = d->ldq; a.cache = d->cache; a.row = d->row; a.H = d->H; a.G = d->G; a.dn = d->dn; a.dv = d->dv;
     a.pos0 = d->pos0; a.T = d->T; a.window = d->window; a.scale = d->scale; a.lambda = d->lambda; a.sub_norm = d->sub_norm; a.eps = d->eps; a.out_scale = d->out_scale;
-    a.splits = d->scratch ? window_splits(d->T, d->H, d->G, window_keys(d->pos0, d->T, d->window)) : 1;
+    if ((d->mask_mode != NTK_MASK_SLIDING && d->mask_mode != NTK_MASK_CHUNKS) || d->softcap < 0.0f) return NTK_E_SHAPE;
+    a.chunks = d->mask_mode == NTK_MASK_CHUNKS; a.softcap = d->softcap; a.sink = d->sink;
+    a.splits = d->scratch ? window_splits(d->T, d->H, d->G, window_keys(d->pos0, d->T, d->window, a.chunks)) : 1;
     a.scratch = d->scratch;
     a.rel = d->rel; a.bucket_of = d->bucket_of; a.n_dist = d->n_dist;
     if (a.rel && (!a.bucket_of || a.n_dist <= 0)) return NTK_E_NULL;
