@@ -60,10 +60,11 @@ def parse():
     ap.add_argument("--cpu-tokens", type=int, default=128, help="-n of the reference CLI run that is the CPU baseline (BASELINE config 1: 128)")
     ap.add_argument("--no-also", action="store_true", help="skip the other BASELINE configurations (8B Q4_K_M, 70B Q4_K_M, 70B Q6_K, 8B Q8_0 behind 3900- and 32768-token prompts)")
     ap.add_argument("--no-pmc-note", action="store_true")
-    ap.add_argument("--family", default="", choices=["", "fabolorn", "nizorax", "tubazen"],
+    ap.add_argument("--family", default="", choices=["", "fabolorn", "nizorax", "tubazen", "fifotar"],
                     help="instead of the default workload: prompt and decode throughput of a layer-list family on synthetic real-sized layers; beside it, fabolorn: the "
                          "Llama path at equal width / heads / active feed-forward width (F16 and Q8_0), nizorax: the fabolorn family at the same preset, tubazen: the nizorax "
-                         "family at the same preset with the dense feed-forward in every layer; one JSON line of its own")
+                         "family at the same preset with the dense feed-forward in every layer, fifotar: the tubazen family at the same preset and number of layers; "
+                         "one JSON line of its own")
     ap.add_argument("--family-size", default="lite", choices=["tiny", "lite", "mid"])
     ap.add_argument("--family-no-compare", action="store_true", help="skip the runs beside the family (a profile of the family's kernels alone)")
     ap.add_argument("--family-layers", type=int, default=2)
@@ -425,12 +426,14 @@ def time_folder(args, cfg, prompt, ctx):
 
 
 def run_family(args):
-    """--family fabolorn | nizorax | tubazen: a synthetic model folder of `--family-layers` real-sized layers (ntransformer_amd/synth_folder.py), a prompt pass of
+    """--family fabolorn | nizorax | tubazen | fifotar: a synthetic model folder of `--family-layers` real-sized layers (ntransformer_amd/synth_folder.py), a prompt pass of
     --prompt-bench tokens (second of two runs) and --steps decoded tokens behind it through the slot cache.  Beside it, unless --family-no-compare:
     fabolorn -- the Llama path with the same width, heads (head size 128), layers, vocabulary and ACTIVE feed-forward width (top x ff + shared ff) as
     F16 and as Q8_0, same prompt and decode; nizorax -- the Fabolorn family (the closest model: same layer stack, slots and products) at the same preset;
     tubazen -- the Nizorax family (the closest model: attention layers beside recurrent ones) at the same preset with the dense feed-forward in every layer
-    (equal feed-forward bytes: three matrices here, two there)."""
+    (equal feed-forward bytes: three matrices here, two there); fifotar -- the Tubazen family (the closest model: attention beside a delta-rule recurrence, a
+    gated dense feed-forward of the same three matrices) at the same preset and number of layers (its layers go attention, delta, latent attention, delta:
+    --family-layers 4 shows every mixer)."""
     import numpy as np
     from ntransformer_amd import _lib, synth_folder
     from ntransformer_amd import engine as E
@@ -441,7 +444,11 @@ def run_family(args):
     rng = np.random.Generator(np.random.Philox(key=[20260925, 7]))
     prompt = [int(t) for t in rng.integers(0, p["vocab"], T)]
     out = {}
-    if args.family == "tubazen":
+    if args.family == "fifotar":
+        out["fifotar"] = time_folder(args, synth_folder.fifotar_config(args.family_size, args.family_layers), prompt, ctx)
+        if not args.family_no_compare:
+            out["tubazen"] = time_folder(args, synth_folder.tubazen_config(args.family_size, args.family_layers, positions=max(ctx, 2048)), prompt, ctx)
+    elif args.family == "tubazen":
         out["tubazen"] = time_folder(args, synth_folder.tubazen_config(args.family_size, args.family_layers, positions=max(ctx, 2048)), prompt, ctx)
         if not args.family_no_compare:
             out["nizorax"] = time_folder(args, synth_folder.nizorax_config(args.family_size, args.family_layers, dense_only=True), prompt, ctx)

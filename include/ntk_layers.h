@@ -273,6 +273,9 @@ typedef struct ntk_gated_recurrence_desc {
     int H, dn, dv;
     float q_scale;
     int pos0, T;
+    float* scratch;   /* F32 [>= ntk_gated_recurrence_scratch(T, H, dn, dv, az != NULL)]: portions of more than a few tokens form their per-token vectors in a launch
+                         of their own, once per head instead of once per workgroup, and long portions are walked in segments side by side (their states and
+                         what the outputs are still owed are settled by two more launches); NULL: always inside the walk, tokens strictly in turn */
     /* ---- the delta rule with one gate per head (all zero / NULL: the forms above) ----
      * G > 0: q and k have G heads [T][G][dn] and state head h reads head h / (H / G) of them (H % G == 0).
      * unit_q / unit_k != 0: q (before q_scale) / the written key k are divided by sqrt(sum x^2 + unit_eps) over the head's dn entries.
@@ -283,9 +286,6 @@ typedef struct ntk_gated_recurrence_desc {
      * Any of these makes every portion form its vectors in a launch of its own: scratch must hold ntk_gated_recurrence_scratch_ex(d) floats. */
     int G, unit_q, unit_k, head_gates, write_gated;
     const float* decay_rates;
-    float* scratch;   /* F32 [>= ntk_gated_recurrence_scratch(T, H, dn, dv, az != NULL)]: portions of more than a few tokens form their per-token vectors in a launch
-                         of their own, once per head instead of once per workgroup, and long portions are walked in segments side by side (their states and
-                         what the outputs are still owed are settled by two more launches); NULL: always inside the walk, tokens strictly in turn */
 } ntk_gated_recurrence_desc;
 size_t ntk_gated_recurrence_scratch(int T, int H, int dn, int dv, int removal);
 size_t ntk_gated_recurrence_scratch_ex(const ntk_gated_recurrence_desc* d);   /* from d's T, H, dn, dv, az and the per-head options */

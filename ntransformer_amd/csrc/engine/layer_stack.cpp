@@ -340,7 +340,7 @@ int LayerStackModel::parse(const ModelFolder& f) {
         for (auto& S : layers_) {
             if (S.mixer != kMixWindow || !S.att.v_mix) continue;
             if (!first) { S.att.v_source = true; first = &S.att; continue; }
-            if (S.att.kv_heads * S.att.vdim != first->kv_heads * first->vdim) return fail(NTK_E_FORMAT, "config: attention layers that blend their values must have the same kv_heads * vdim");
+            if (S.att.kv_heads != first->kv_heads || S.att.vdim != first->vdim) return fail(NTK_E_FORMAT, "config: attention layers that blend their values must have the same kv_heads and vdim");
         }
     }
     if (has_loop_) {

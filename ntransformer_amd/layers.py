@@ -23,14 +23,25 @@ class DenseDesc(C.Structure):
 
 
 class Rotary(C.Structure):
-    _fields_ = [("freq", C.c_void_p), ("mag", C.c_float), ("dims", C.c_int)]
+    _fields_ = [("freq", C.c_void_p), ("mag", C.c_float), ("dims", C.c_int), ("layout", C.c_int)]
+
+
+ROT_NEIGHBOURS, ROT_HALVES = 0, 1
+MASK_SLIDING, MASK_CHUNKS = 0, 1
+
+
+class WindowPrepareDesc(C.Structure):
+    _fields_ = [("cache", C.c_void_p), ("row", C.c_int), ("q", C.c_void_p), ("ldq", C.c_int), ("k", C.c_void_p), ("ldk", C.c_int), ("v", C.c_void_p), ("ldv", C.c_int),
+                ("H", C.c_int), ("G", C.c_int), ("maps", C.c_int), ("dn", C.c_int), ("dv", C.c_int), ("rot", C.POINTER(Rotary)),
+                ("qb", C.c_void_p), ("kb", C.c_void_p), ("vb", C.c_void_p), ("temp_coef", C.c_float), ("temp_every", C.c_double),
+                ("v_other", C.c_void_p), ("ld_other", C.c_int), ("v_blend", C.c_float), ("v_keep", C.c_void_p), ("ld_keep", C.c_int), ("pos0", C.c_int), ("T", C.c_int)]
 
 
 class WindowAttentionDesc(C.Structure):
     _fields_ = [("out", C.c_void_p), ("ldo", C.c_int), ("q", C.c_void_p), ("ldq", C.c_int), ("cache", C.c_void_p), ("row", C.c_int),
                 ("H", C.c_int), ("G", C.c_int), ("maps", C.c_int), ("dn", C.c_int), ("dv", C.c_int), ("pos0", C.c_int), ("T", C.c_int), ("window", C.c_int),
                 ("scale", C.c_float), ("lam", C.c_float), ("sub_norm", C.c_int), ("eps", C.c_float), ("out_scale", C.c_float), ("scratch", C.c_void_p),
-                ("rel", C.c_void_p), ("bucket_of", C.c_void_p), ("n_dist", C.c_int)]
+                ("rel", C.c_void_p), ("bucket_of", C.c_void_p), ("n_dist", C.c_int), ("mask_mode", C.c_int), ("softcap", C.c_float), ("sink", C.c_int)]
 
 
 class GatedSeamDesc(C.Structure):
@@ -43,10 +54,11 @@ class GatedRecurrenceDesc(C.Structure):
     _fields_ = [("out", C.c_void_p), ("ldo", C.c_int), ("q", C.c_void_p), ("ldq", C.c_int), ("k", C.c_void_p), ("ldk", C.c_int), ("v", C.c_void_p), ("ldv", C.c_int),
                 ("wz", C.c_void_p), ("ldw", C.c_int), ("wb", C.c_void_p), ("decay_form", C.c_int), ("decay_param", C.c_float),
                 ("az", C.c_void_p), ("lda", C.c_int), ("ab", C.c_void_p), ("unit_eps", C.c_float), ("state", C.c_void_p),
-                ("H", C.c_int), ("dn", C.c_int), ("dv", C.c_int), ("q_scale", C.c_float), ("pos0", C.c_int), ("T", C.c_int), ("scratch", C.c_void_p)]
+                ("H", C.c_int), ("dn", C.c_int), ("dv", C.c_int), ("q_scale", C.c_float), ("pos0", C.c_int), ("T", C.c_int), ("scratch", C.c_void_p),
+                ("G", C.c_int), ("unit_q", C.c_int), ("unit_k", C.c_int), ("head_gates", C.c_int), ("write_gated", C.c_int), ("decay_rates", C.c_void_p)]
 
 
-DECAY_GIVEN, DECAY_SIGMOID_ROOT, DECAY_EXP_SIGMOID = 0, 1, 2
+DECAY_GIVEN, DECAY_SIGMOID_ROOT, DECAY_EXP_SIGMOID, DECAY_EXP_SOFTPLUS = 0, 1, 2, 3
 
 
 class RouteDesc(C.Structure):
@@ -105,6 +117,14 @@ def _bind():
     L.ntk_gated_recurrence_scratch.argtypes = [i, i, i, i, i]
     L.ntk_gated_recurrence_scratch.restype = C.c_size_t
     L.ntk_glu_cubic.argtypes = [vp, vp, i, i, i, f, f, f, f, vp]
+    L.ntk_rms_seam.argtypes = [vp, i, vp, i, vp, i, vp, f, vp, i, i, f, vp]
+    L.ntk_causal_conv_act.argtypes = [vp, i, vp, i, vp, vp, i, i, i, i, i, vp]
+    L.ntk_softcap_rows.argtypes = [vp, i, f, i, i, vp]
+    L.ntk_head_gate.argtypes = [vp, i, vp, i, i, i, i, vp]
+    L.ntk_latent_unfold_value_ex.argtypes = [vp, i, vp, vp, i, vp, i, i, i, i, i, i, vp]
+    L.ntk_window_prepare_ex.argtypes = [C.POINTER(WindowPrepareDesc), vp]
+    L.ntk_gated_recurrence_scratch_ex.argtypes = [C.POINTER(GatedRecurrenceDesc)]
+    L.ntk_gated_recurrence_scratch_ex.restype = C.c_size_t
     L._layers_bound = True
     return L
 
@@ -176,7 +196,7 @@ def rmsnorm_offset(x: np.ndarray, w1: np.ndarray, w2: Optional[np.ndarray], eps:
 
 
 def latent_prepare(kv: np.ndarray, norm_w: np.ndarray, eps: float, kv_rank: int, rot_dim: int, q: Optional[np.ndarray], heads: int, freq: np.ndarray, mag: float,
-                   dims: int, pos0: int, cache: Optional[np.ndarray] = None, cache_rows: Optional[int] = None):
+                   dims: int, pos0: int, cache: Optional[np.ndarray] = None, cache_rows: Optional[int] = None, layout: int = ROT_NEIGHBOURS):
     """-> (cache [rows, kv_rank + rot_dim] with rows pos0.. filled, q rotated)"""
     L = _bind()
     T, row = kv.shape[0], kv_rank + rot_dim
@@ -185,7 +205,7 @@ def latent_prepare(kv: np.ndarray, norm_w: np.ndarray, eps: float, kv_rank: int,
     kb, nb, fb = _f(kv), _f(norm_w), DeviceBuffer.from_numpy(np.ascontiguousarray(freq, np.float64))
     qb = _f(q) if q is not None else None
     qd = q.shape[1] // heads if q is not None else rot_dim
-    rot = Rotary(fb.ptr, mag, dims)
+    rot = Rotary(fb.ptr, mag, dims, layout)
     check(L.ntk_latent_prepare(cb.ptr, row, kb.ptr, kv.shape[1], nb.ptr, eps, kv_rank, rot_dim, qb.ptr if qb else None, q.shape[1] if q is not None else 0, heads, qd,
                                C.byref(rot), pos0, T, None), "ntk_latent_prepare")
     return cb.numpy(np.float32, n * row).reshape(n, row), (qb.numpy(np.float32, q.size).reshape(q.shape) if qb else None)
@@ -221,14 +241,16 @@ def latent_fold_query(q: np.ndarray, w_uk: np.ndarray, heads: int, dn: int, dr: 
     return out.numpy(np.float32, T * heads * (R + dr)).reshape(T, heads * (R + dr))
 
 
-def latent_unfold_value(lat: np.ndarray, w_uv: np.ndarray, heads: int, gate: Optional[np.ndarray] = None, dtype: str = "float32") -> np.ndarray:
+def latent_unfold_value(lat: np.ndarray, w_uv: np.ndarray, heads: int, gate: Optional[np.ndarray] = None, dtype: str = "float32", head_gate: bool = False) -> np.ndarray:
+    """head_gate: gate [T, heads] (one number per head) instead of [T, heads * dv]"""
     L = _bind()
     T, R = lat.shape[0], w_uv.shape[1]
     dv = w_uv.shape[0] // heads
     lb, (wb, wdt) = _f(lat), weight_buffer(w_uv, dtype)
     gb = _f(gate) if gate is not None else None
     out = DeviceBuffer.zeros(T * heads * dv * 4)
-    check(L.ntk_latent_unfold_value(out.ptr, heads * dv, lb.ptr, wb.ptr, wdt, gb.ptr if gb else None, heads * dv, T, heads, dv, R, None), "ntk_latent_unfold_value")
+    check(L.ntk_latent_unfold_value_ex(out.ptr, heads * dv, lb.ptr, wb.ptr, wdt, gb.ptr if gb else None, gate.shape[1] if gate is not None else 0, int(head_gate), T, heads,
+                                       dv, R, None), "ntk_latent_unfold_value")
     return out.numpy(np.float32, T * heads * dv).reshape(T, heads * dv)
 
 
@@ -364,7 +386,7 @@ def window_prepare_biased(q, k, v, H: int, G: int, dn: int, dv: int, pos0: int, 
 
 def window_attention(q: np.ndarray, cache: np.ndarray, H: int, G: int, maps: int, dn: int, dv: int, pos0: int, window: int, scale: float, lam: float = 0.0,
                      sub_norm: bool = False, eps: float = 1e-6, out_scale: float = 1.0, split: bool = True, rel: Optional[np.ndarray] = None,
-                     bucket_of: Optional[np.ndarray] = None) -> np.ndarray:
+                     bucket_of: Optional[np.ndarray] = None, chunks: bool = False, softcap: float = 0.0, sink: bool = False) -> np.ndarray:
     """q [T, H * maps * dn] (rotated), cache rows [G][maps][dn] keys | [G][dv] values; split: long key ranges of few rows may be cut into merged parts;
     rel [buckets, H] with bucket_of [distances]: a bias by distance on the scaled score"""
     L = _bind()
@@ -377,6 +399,7 @@ def window_attention(q: np.ndarray, cache: np.ndarray, H: int, G: int, maps: int
     if rel is not None:
         rb, bb = _f(rel), _i(bucket_of)
         d.rel, d.bucket_of, d.n_dist = rb.ptr, bb.ptr, len(bucket_of)
+    d.mask_mode, d.softcap, d.sink = (MASK_CHUNKS if chunks else MASK_SLIDING), softcap, int(sink)
     check(L.ntk_window_attention(C.byref(d), None), "ntk_window_attention")
     return out.numpy(np.float32, T * H * dv).reshape(T, H * dv)
 
@@ -493,7 +516,8 @@ def gated_seam(x, y=None, g=None, yb=None, gb=None, hist=None, coef=None, norm=N
 
 
 def gated_recurrence(q, k, v, wz, H: int, dn: int, dv: int, pos0: int, decay_form: int = DECAY_GIVEN, decay_param: float = 1.0, wb=None, az=None, ab=None,
-                     unit_eps: float = 1e-6, q_scale: float = 1.0, state: Optional[np.ndarray] = None, prepass: bool = True):
+                     unit_eps: float = 1e-6, q_scale: float = 1.0, state: Optional[np.ndarray] = None, prepass: bool = True, G: int = 0, unit_q: bool = False,
+                     unit_k: bool = False, head_gates: bool = False, write_gated: bool = False, decay_rates=None):
     """-> (out [T, H * dv], state [H, dn, dv]); az: the removal rate's raw projection (None: no removal term); state: what an earlier portion left (ignored when
     pos0 == 0; by default full of NaN so that a read at the start would show); prepass: give the scratch that lets longer portions form their per-token vectors
     in a launch of their own"""
@@ -506,7 +530,9 @@ def gated_recurrence(q, k, v, wz, H: int, dn: int, dv: int, pos0: int, decay_for
     d = GatedRecurrenceDesc(out.ptr, H * dv, qb.ptr, q.shape[1], kb.ptr, k.shape[1], vb.ptr, v.shape[1], zb.ptr, wz.shape[1], wbb.ptr if wbb else None, decay_form,
                             decay_param, azb.ptr if azb else None, az.shape[1] if az is not None else 0, abb.ptr if abb else None, unit_eps, sb.ptr, H, dn, dv, q_scale,
                             pos0, T, None)
-    ns = int(L.ntk_gated_recurrence_scratch(T, H, dn, dv, int(az is not None))) if prepass else 0
+    rb = _f(decay_rates) if decay_rates is not None else None
+    d.G, d.unit_q, d.unit_k, d.head_gates, d.write_gated, d.decay_rates = G, int(unit_q), int(unit_k), int(head_gates), int(write_gated), rb.ptr if rb else None
+    ns = int(L.ntk_gated_recurrence_scratch_ex(C.byref(d))) if prepass else 0
     scr = DeviceBuffer.from_numpy(np.full(ns, np.nan, np.float32)) if ns else None
     if scr:
         d.scratch = scr.ptr
@@ -522,3 +548,67 @@ def glu_cubic(gu: np.ndarray, ff: int, alpha: float, cubic: float, limit: float 
     out = DeviceBuffer.zeros(rows * ff * 4)
     check(L.ntk_glu_cubic(out.ptr, gb.ptr, gu.shape[1], rows, ff, limit, alpha, cubic, up_offset, None), "ntk_glu_cubic")
     return out.numpy(np.float32, rows * ff).reshape(rows, ff)
+
+
+def window_prepare_ex(q, k, v, H: int, G: int, dn: int, dv: int, pos0: int, freq=None, dims: int = 0, layout: int = ROT_NEIGHBOURS, v_other=None, v_blend: float = 0.0,
+                      keep: bool = False, cache: Optional[np.ndarray] = None, cache_rows: Optional[int] = None):
+    """one score map: rotation by `layout`, values blended with v_other [T, G * dv] on their way into the cache rows -> (cache, q, the values as they came if keep)"""
+    L = _bind()
+    T, row = q.shape[0], G * (dn + dv)
+    n = cache_rows or (pos0 + T)
+    cb = _f(cache) if cache is not None else DeviceBuffer.zeros(n * row * 4)
+    qd, kd, vd = _f(q), _f(k), _f(v)
+    fb = DeviceBuffer.from_numpy(np.ascontiguousarray(freq if freq is not None and len(freq) else [0.0], np.float64))
+    rot = Rotary(fb.ptr, 1.0, dims, layout)
+    ob = _f(v_other) if v_other is not None else None
+    kb = DeviceBuffer.zeros(T * G * dv * 4) if keep else None
+    d = WindowPrepareDesc()
+    d.cache, d.row, d.q, d.ldq, d.k, d.ldk, d.v, d.ldv = cb.ptr, row, qd.ptr, q.shape[1], kd.ptr, k.shape[1], vd.ptr, v.shape[1]
+    d.H, d.G, d.maps, d.dn, d.dv, d.rot, d.temp_every, d.pos0, d.T = H, G, 1, dn, dv, C.pointer(rot), 1.0, pos0, T
+    if ob:
+        d.v_other, d.ld_other, d.v_blend = ob.ptr, G * dv, v_blend
+    if kb:
+        d.v_keep, d.ld_keep = kb.ptr, G * dv
+    check(L.ntk_window_prepare_ex(C.byref(d), None), "ntk_window_prepare_ex")
+    return (cb.numpy(np.float32, n * row).reshape(n, row), qd.numpy(np.float32, q.size).reshape(q.shape),
+            kb.numpy(np.float32, T * G * dv).reshape(T, G * dv) if kb else None)
+
+
+def rms_seam(x: np.ndarray, w: Optional[np.ndarray], eps: float, add_y: Optional[np.ndarray] = None, add_w: Optional[np.ndarray] = None, mult: float = 1.0):
+    """x += mult * rms(add_y) * add_w (if add_y), h = rms(x) * w (if w) -> (x, h or None)"""
+    L = _bind()
+    T, n = x.shape
+    xb = _f(x)
+    yb, awb, wb = (_f(a) if a is not None else None for a in (add_y, add_w, w))
+    hb = DeviceBuffer.zeros(T * n * 4) if w is not None else None
+    check(L.ntk_rms_seam(hb.ptr if hb else None, n, xb.ptr, n, yb.ptr if yb else None, n, awb.ptr if awb else None, mult, wb.ptr if wb else None, T, n, eps, None), "ntk_rms_seam")
+    return xb.numpy(np.float32, T * n).reshape(T, n), (hb.numpy(np.float32, T * n).reshape(T, n) if hb else None)
+
+
+def causal_conv_act(x: np.ndarray, w: np.ndarray, pos0: int, state: Optional[np.ndarray] = None, act: int = 1, n: Optional[int] = None):
+    """x [T, >= n] (the first n columns are the channels), w [n, taps], state [taps - 1, n] (by default full of NaN) -> (y [T, n], state)"""
+    L = _bind()
+    T, taps = x.shape[0], w.shape[1]
+    n = n or w.shape[0]
+    xb, wb = _f(x), _f(w)
+    sb = _f(state) if state is not None and np.size(state) else DeviceBuffer.from_numpy(np.full(max(taps - 1, 1) * n, np.nan, np.float32))
+    yb = DeviceBuffer.zeros(T * n * 4)
+    check(L.ntk_causal_conv_act(yb.ptr, n, xb.ptr, x.shape[1], wb.ptr, sb.ptr, taps, act, pos0, T, n, None), "ntk_causal_conv_act")
+    return yb.numpy(np.float32, T * n).reshape(T, n), sb.numpy(np.float32, max(taps - 1, 1) * n).reshape(max(taps - 1, 1), n)[:taps - 1]
+
+
+def softcap_rows(x: np.ndarray, cap: float) -> np.ndarray:
+    L = _bind()
+    T, n = x.shape
+    xb = _f(x)
+    check(L.ntk_softcap_rows(xb.ptr, n, cap, T, n, None), "ntk_softcap_rows")
+    return xb.numpy(np.float32, T * n).reshape(T, n)
+
+
+def head_gate(y: np.ndarray, g: np.ndarray, H: int) -> np.ndarray:
+    """y [T, H * dv] times sigmoid(g [T, H]) per head"""
+    L = _bind()
+    T, dv = y.shape[0], y.shape[1] // H
+    yb, gb = _f(y), _f(g)
+    check(L.ntk_head_gate(yb.ptr, y.shape[1], gb.ptr, g.shape[1], T, H, dv, None), "ntk_head_gate")
+    return yb.numpy(np.float32, y.size).reshape(y.shape)

@@ -179,9 +179,66 @@ def tubazen_shapes(cfg: dict, buckets: int = 32, rank: int = 64) -> Dict[str, Tu
     return s
 
 
+def fifotar_config(preset: str, layers: int = 4, mlp_everywhere: bool = True) -> dict:
+    """the scaled family at the preset's width, heads and vocabulary: chunked attention (four query heads per key/value head, chunks of the preset's window,
+    capped scores, blended values), the per-head delta rule (two value heads per key head, keys and values of the preset's sizes, four taps) and latent
+    attention (the preset's ranks) in the order attention, delta, latent, delta; the clipped gated feed-forward with the bytes of the gated family's"""
+    p = PRESETS[preset]
+    H, dn, dv = p["heads"], p["dim"], p["vdim"]
+    ff = (p["top"] * p["ff"] + p["shared_ff"]) * 2 // 3
+    ff -= ff % 64
+    ls = []
+    for k in range(layers):
+        if k % 4 == 0:
+            mx = {"heads": H, "kv_heads": max(H // 4, 1), "dim": dn, "vdim": dv, "scale": 1.0 / math.sqrt(dn), "softcap": 50.0, "mask": {"size": p["window"]}, "v_mix": True}
+            t = "attention"
+        elif k % 4 == 2:
+            mx = {"heads": H, "dim": dn, "rot_dim": p["rot_dim"], "vdim": dv, "kv_rank": p["kv_rank"], "q_rank": p["q_rank"], "scale": 1.0 / math.sqrt(dn + p["rot_dim"]),
+                  "rot": {"base": 1000000.0, "dims": p["rot_dim"], "scaling": {"factor": 8.0, "original": 4096, "fast": 16.0, "slow": 2.0}}}
+            t = "latent_attention"
+        else:
+            mx = {"heads": H, "kv_heads": max(H // 2, 1), "dim": dn, "vdim": dv, "conv": 4}
+            t = "delta"
+        has_mlp = mlp_everywhere or t != "delta"
+        ls.append({"type": t, "mixer": mx, "mlp": {"kind": "dense", "ff": max(ff, 64), "limit": 7.0} if has_mlp else None})
+    return {"architecture": "Fifotar", "layers": ls, "norm": {"eps": 1e-5}, "embedding": {"scale": math.sqrt(p["width"])}, "residual_mult": 0.5, "logit_softcap": 30.0,
+            "vocab": p["vocab"], "width": p["width"]}
+
+
+def fifotar_shapes(cfg: dict) -> Dict[str, Tuple[int, ...]]:
+    W, V = cfg["width"], cfg["vocab"]
+    s: Dict[str, Tuple[int, ...]] = {"embed": (V, W), "final.norm": (W,)}
+    for i, L in enumerate(cfg["layers"]):
+        p, mx, ml = "l%d." % i, L["mixer"], L.get("mlp")
+        for nm in ("norm1", "norm1b") + (("norm2", "norm2b") if ml else ()):
+            s[p + nm] = (W,)
+        q = p + "mix."
+        H, dn, dv = mx["heads"], mx["dim"], mx["vdim"]
+        if L["type"] == "attention":
+            G = mx.get("kv_heads", H)
+            s[q + "q"], s[q + "k"], s[q + "v"], s[q + "g"], s[q + "o"] = (H * dn, W), (G * dn, W), (G * dv, W), (H * dv, W), (W, H * dv)
+            if mx.get("v_mix"):
+                s[q + "vmix"] = ()
+        elif L["type"] == "latent_attention":
+            dr, R, Q = mx["rot_dim"], mx["kv_rank"], mx["q_rank"]
+            s[q + "dq"], s[q + "dq.norm"], s[q + "uq"] = (Q, W), (Q,), (H * (dn + dr), Q)
+            s[q + "dkv"], s[q + "dkv.norm"], s[q + "uk"], s[q + "uv"] = (R + dr, W), (R,), (H * dn, R), (H * dv, R)
+            s[q + "g"], s[q + "o"] = (H, W), (W, H * dv)
+        else:
+            G, K = mx.get("kv_heads", H), mx.get("conv", 1)
+            for nm, rows in (("q", G * dn), ("k", G * dn), ("v", H * dv)):
+                s[q + nm], s[q + nm + ".conv"] = (rows, W), (rows, K)
+            s[q + "b"], s[q + "a"], s[q + "A_log"], s[q + "dt_bias"] = (H, W), (H, W), (H,), (H,)
+            s[q + "norm"], s[q + "g"], s[q + "o"] = (dv,), (H * dv, W), (W, H * dv)
+        if ml:
+            s[p + "mlp.gate"], s[p + "mlp.up"], s[p + "mlp.down"] = (ml["ff"], W), (ml["ff"], W), (W, ml["ff"])
+    return s
+
+
 def shapes_of(cfg: dict) -> Dict[str, Tuple[int, ...]]:
     arch = cfg.get("architecture")
-    return nizorax_shapes(cfg) if arch == "Nizorax" else tubazen_shapes(cfg) if arch == "Tubazen" else fabolorn_shapes(cfg)
+    return (nizorax_shapes(cfg) if arch == "Nizorax" else tubazen_shapes(cfg) if arch == "Tubazen" else fifotar_shapes(cfg) if arch == "Fifotar" else
+            fabolorn_shapes(cfg))
 
 
 def _bf16(a: np.ndarray) -> np.ndarray:
@@ -211,6 +268,8 @@ def write_folder(folder: str, cfg: dict, seed: int = 20260925) -> int:
             n = int(np.prod(shp))
             if len(shp) == 0 or name.endswith(".dwa"):       # a norm's slope around one; depth weights: an average over the results so far
                 vals = (1.0 + 0.1 * pool[:1]) if len(shp) == 0 else (1.0 / n + 0.01 * pool[:n])
+                if name.endswith(".vmix"):                    # a blend weight between zero and one
+                    vals = np.array([0.5], np.float32)
                 f.write(_bf16(vals).tobytes())
                 continue
             if len(shp) == 1:
@@ -219,6 +278,8 @@ def write_folder(folder: str, cfg: dict, seed: int = 20260925) -> int:
                     around_one = name.rsplit(".", 1)[-1] in ("norm", "norm1", "norm2")
                 if cfg.get("architecture") == "Nizorax":     # layer-norm weights around one, biases / lambda vectors / activation numbers small
                     around_one = name.rsplit(".", 1)[-1] in ("norm", "norm1", "norm2", "norm1b", "norm2b")
+                if cfg.get("architecture") == "Fifotar":     # every norm weight is stored plain; decay rates and biases small
+                    around_one = "norm" in name.rsplit(".", 1)[-1]
                 vals = 0.1 * pool[:n] + (1.0 if around_one else 0.0)
                 f.write(_bf16(vals).tobytes())
                 continue

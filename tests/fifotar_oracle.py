@@ -57,6 +57,26 @@ def sink_softmax(s):
     return e / (math.exp(-m) + e.sum())
 
 
+def attend(q, k, v, pos0, scale, size=None, cap=None, sink=True):
+    """q [T, H, dn] at positions pos0 ..; k [P, G, dn], v [P, G, dv] of positions 0 .. P - 1 -> [T, H, dv]"""
+    T, H, _ = q.shape
+    G = k.shape[1]
+    out = np.zeros((T, H, v.shape[2]), F)
+    for t in range(T):
+        p = pos0 + t
+        js = [j for j in range(p + 1) if sees_chunk(p, j, size)]
+        for hh in range(H):
+            g = hh // (H // G)
+            s = capped((k[js, g] @ q[t, hh]) * scale, cap)
+            if sink:
+                wts = sink_softmax(s)
+            else:
+                e = np.exp(s - s.max())
+                wts = e / e.sum()
+            out[t, hh] = wts @ v[js, g]
+    return out
+
+
 def chunked_attention(h, w, pre, mx, pos0=0, past=None, v_first=None):
     """h [T, W] at positions pos0 ..; past = (k, v) of earlier positions; v_first [T, G, dv]: the first blending layer's values of the same tokens (None in
     that layer itself or without blending) -> (out [T, W], (k, v) so far, this layer's raw values [T, G, dv])"""
@@ -71,15 +91,7 @@ def chunked_attention(h, w, pre, mx, pos0=0, past=None, v_first=None):
         v = (1.0 - lam) * v + lam * v_first
     if past is not None:
         k, v = np.concatenate([past[0], k]), np.concatenate([past[1], v])
-    size = (mx.get("mask") or {}).get("size")
-    out = np.zeros((T, H, dv), F)
-    for t in range(T):
-        p = pos0 + t
-        js = [j for j in range(p + 1) if sees_chunk(p, j, size)]
-        for hh in range(H):
-            g = hh // (H // G)
-            s = capped((k[js, g] @ q[t, hh]) * mx["scale"], mx.get("softcap"))
-            out[t, hh] = sink_softmax(s) @ v[js, g]
+    out = attend(q, k, v, pos0, mx["scale"], (mx.get("mask") or {}).get("size"), mx.get("softcap"))
     out = out.reshape(T, H * dv) * sigmoid(h @ w[pre + "g"].T)
     return out @ w[pre + "o"].T, (k, v), v_own
 
@@ -243,6 +255,16 @@ def forward(cfg, w, tokens, seq=None, layers_out=None):
     z = rms(x, w["final.norm"], eps) @ E.T
     cap = cfg.get("logit_softcap")
     return (cap * np.tanh(z / cap) if cap else z), seq
+
+
+def greedy(cfg, w, prompt, n):
+    """n tokens, each the argmax of the last position's logits"""
+    logits, seq = forward(cfg, w, prompt)
+    out = []
+    for _ in range(n):
+        out.append(int(np.argmax(logits[-1])))
+        logits, seq = forward(cfg, w, [out[-1]], seq)
+    return out
 
 
 # ---------------------------------------------------------------------------------------------------------------- configurations and folders
