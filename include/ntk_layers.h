@@ -286,6 +286,9 @@ typedef struct ntk_gated_recurrence_desc {
      * Any of these makes every portion form its vectors in a launch of its own: scratch must hold ntk_gated_recurrence_scratch_ex(d) floats. */
     int G, unit_q, unit_k, head_gates, write_gated;
     const float* decay_rates;
+    /* conv_w != NULL (T == 1 only: a decoded token): q, k, v are RAW projections that first pass the short causal convolution + silu of ntk_causal_conv_act inside
+     * the pre-pass's launch -- conv_w F32 [2 G dn + H dv][conv_taps] and the carried inputs conv_state [conv_taps - 1][2 G dn + H dv], channels in the order q | k | v. */
+    const float* conv_w; float* conv_state; int conv_taps;
 } ntk_gated_recurrence_desc;
 size_t ntk_gated_recurrence_scratch(int T, int H, int dn, int dv, int removal);
 size_t ntk_gated_recurrence_scratch_ex(const ntk_gated_recurrence_desc* d);   /* from d's T, H, dn, dv, az and the per-head options */

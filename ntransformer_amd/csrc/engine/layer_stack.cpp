@@ -1018,9 +1018,15 @@ int LayerStackModel::run_gated_delta(const StackLayer& L, float* state, int T, i
     const GatedDeltaMixer& m = L.gdl;
     const int W = info_.width, na = (int)m.in.out_f, nc = m.channels(), hv = m.heads * m.vdim;
     LS_TRY(ntk_dense_linear(a_, na, h1_, W, m.in.ptr, m.in.dtype, T, na, W, 0, stream_));
-    LS_TRY(ntk_causal_conv_act(cv_, nc, a_, na, m.conv, state + m.recurrent_floats(), m.taps, 1, pos0, T, nc, stream_));
     ntk_gated_recurrence_desc d{};
-    d.out = att_; d.ldo = hv; d.q = cv_; d.ldq = nc; d.k = cv_ + m.k_off; d.ldk = nc; d.v = cv_ + m.v_off; d.ldv = nc;
+    if (T == 1) {   // a decoded token: the convolutions run inside the recurrence's pre-pass
+        d.q = a_; d.ldq = na; d.k = a_ + m.k_off; d.ldk = na; d.v = a_ + m.v_off; d.ldv = na;
+        d.conv_w = m.conv; d.conv_state = state + m.recurrent_floats(); d.conv_taps = m.taps;
+    } else {
+        LS_TRY(ntk_causal_conv_act(cv_, nc, a_, na, m.conv, state + m.recurrent_floats(), m.taps, 1, pos0, T, nc, stream_));
+        d.q = cv_; d.ldq = nc; d.k = cv_ + m.k_off; d.ldk = nc; d.v = cv_ + m.v_off; d.ldv = nc;
+    }
+    d.out = att_; d.ldo = hv;
     d.wz = a_ + m.a_off; d.ldw = na; d.wb = m.dt_bias; d.decay_form = NTK_DECAY_EXP_SOFTPLUS; d.decay_rates = m.rates;
     d.az = a_ + m.b_off; d.lda = na; d.unit_eps = kUnitKeyEps;
     d.G = m.kv_heads; d.unit_q = 1; d.unit_k = 1; d.head_gates = 1; d.write_gated = 1;

@@ -51,6 +51,8 @@ struct RecArgs {
     int G, unit_q, unit_k, head_gates, write_gated;
     const float* decay_rates;
     float* vpacked;                  // [T][H][dv]: values times the removal rate (write_gated); the walk then reads these
+    // a short causal convolution + silu on the raw q, k, v of ONE token inside the pre-pass (conv_w [2 G dn + H dv][taps], the carried inputs conv_state)
+    const float* conv_w; float* conv_state; int conv_taps;
 };
 
 constexpr int kRecFewTokens = 8;  // up to this many tokens (decoding) the walk forms its vectors itself: one launch
@@ -107,6 +109,70 @@ __global__ __launch_bounds__(64) void gated_recurrence_prepare_kernel(const RecA
     if constexpr (DELTA) {
         if (a.write_gated)
             for (int c = lane; c < a.dv; c += 64) a.vpacked[(t * a.H + h) * a.dv + c] = a.v[t * a.ldv + (long long)h * a.dv + c] * ah;
+    }
+}
+
+// One token (decoding) whose q, k, v still have to pass their short convolutions: a workgroup per q / k head.  It convolves the head's q and k channels and the
+// value channels of the state heads that share them (each channel's carried inputs are read, used and shifted by the one thread that owns the channel), then
+// forms the same vectors as the kernel above, with the same sums in the same lane order.
+constexpr int kStepConvTaps = 16;
+__device__ __forceinline__ float conv_step(const float* w, float* state, int taps, int n, int c, float x, int pos0) {
+    float s = 0.0f;
+    for (int j = 0; j + 1 < taps; ++j) {
+        const float hj = pos0 - (taps - 1) + j >= 0 ? state[(long long)j * n + c] : 0.0f;
+        s = fmaf(w[(long long)c * taps + j], hj, s);
+        if (j > 0) state[(long long)(j - 1) * n + c] = hj;
+    }
+    s = fmaf(w[(long long)c * taps + taps - 1], x, s);
+    if (taps > 1) state[(long long)(taps - 2) * n + c] = x;
+    return s / (1.0f + expf(-s));
+}
+
+template <bool DELTA>
+__global__ __launch_bounds__(256) void gated_recurrence_prepare_step_kernel(const RecArgs a) {
+    constexpr int NV = DELTA ? 5 : 3;
+    extern __shared__ float cs[];                        // [dn] q, [dn] k after convolution and silu
+    const int G = a.G > 0 ? a.G : a.H, R = a.H / G, g = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nch = 2 * G * a.dn + a.H * a.dv;           // convolved channels: q | k | v
+    float* qs = cs;
+    float* ks = cs + a.dn;
+    for (int d = threadIdx.x; d < a.dn; d += 256) {
+        qs[d] = conv_step(a.conv_w, a.conv_state, a.conv_taps, nch, g * a.dn + d, a.q[(long long)g * a.dn + d], a.pos0);
+        ks[d] = conv_step(a.conv_w, a.conv_state, a.conv_taps, nch, G * a.dn + g * a.dn + d, a.k[(long long)g * a.dn + d], a.pos0);
+    }
+    __syncthreads();
+    float ss = 0.0f, sq = 0.0f;
+    for (int d = lane; d < a.dn; d += 64) { ss = fmaf(ks[d], ks[d], ss); sq = fmaf(qs[d], qs[d], sq); }
+    const float inv_k = 1.0f / sqrtf(wave_sum(ss) + a.unit_eps);
+    const float qmul = a.unit_q ? a.q_scale / sqrtf(wave_sum(sq) + a.unit_eps) : a.q_scale;
+    const float kmul = a.unit_k ? inv_k : 1.0f;
+    for (int r = wave; r < R; r += 4) {                  // a wave per state head of the group
+        const int h = g * R + r;
+        float* dst = a.packed + (long long)h * NV * a.dn;
+        const long long oc = (long long)h * a.dn;
+        float wh = 1.0f, ah = 0.0f;
+        if (a.head_gates) {
+            wh = decay_of(a.wz[h] + (a.wb ? a.wb[h] : 0.0f), a.decay_form, a.decay_rates ? a.decay_rates[h] : a.decay_param);
+            if constexpr (DELTA) ah = 1.0f / (1.0f + expf(-(a.az[h] + (a.ab ? a.ab[h] : 0.0f))));
+        }
+        for (int d = lane; d < a.dn; d += 64) {
+            const float kk = ks[d];
+            const float w = a.head_gates ? wh : decay_of(a.wz[oc + d] + (a.wb ? a.wb[oc + d] : 0.0f), a.decay_form, a.decay_rates ? a.decay_rates[h] : a.decay_param);
+            dst[d] = qs[d] * qmul;
+            dst[a.dn + d] = kk * kmul;
+            dst[2 * a.dn + d] = w;
+            if constexpr (DELTA) {
+                const float uu = kk * inv_k;
+                const float aa = a.head_gates ? ah : 1.0f / (1.0f + expf(-(a.az[oc + d] + (a.ab ? a.ab[oc + d] : 0.0f))));
+                dst[3 * a.dn + d] = a.write_gated ? uu * w : uu;
+                dst[4 * a.dn + d] = uu * aa;
+            }
+        }
+        for (int c = lane; c < a.dv; c += 64) {
+            const float vv = conv_step(a.conv_w, a.conv_state, a.conv_taps, nch, 2 * G * a.dn + h * a.dv + c, a.v[(long long)h * a.dv + c], a.pos0);
+            a.vpacked[(long long)h * a.dv + c] = (DELTA && a.write_gated) ? vv * ah : vv;
+        }
     }
 }
 
@@ -441,7 +507,11 @@ static int launch_rec_waves(const RecArgs& a0, hipStream_t s) {
     const int ncols = (delta && a.nseg > 1) ? a.dv + a.dn : a.dv;
     const dim3 grid((ncols + CB - 1) / CB, a.H, a.nseg);
     if (a.packed) {
-        if (delta) hipLaunchKernelGGL(gated_recurrence_prepare_kernel<true>, dim3(a.T * a.H), dim3(64), 0, s, a);
+        if (a.conv_w) {
+            const dim3 pgrid(a.G > 0 ? a.G : a.H);
+            if (delta) hipLaunchKernelGGL(gated_recurrence_prepare_step_kernel<true>, pgrid, dim3(256), (size_t)2 * a.dn * sizeof(float), s, a);
+            else hipLaunchKernelGGL(gated_recurrence_prepare_step_kernel<false>, pgrid, dim3(256), (size_t)2 * a.dn * sizeof(float), s, a);
+        } else if (delta) hipLaunchKernelGGL(gated_recurrence_prepare_kernel<true>, dim3(a.T * a.H), dim3(64), 0, s, a);
         else hipLaunchKernelGGL(gated_recurrence_prepare_kernel<false>, dim3(a.T * a.H), dim3(64), 0, s, a);
         const int st = last_launch_status();
         if (st != NTK_OK) return st;
@@ -500,7 +570,7 @@ static int rec_segments(int T, int H, int dn, int dv, bool removal) {
 
 // any of the per-head options: the vectors are always formed by the pre-pass
 static bool rec_needs_prepass(const ntk_gated_recurrence_desc* d) {
-    return d->G > 0 || d->unit_q || d->unit_k || d->head_gates || d->write_gated || d->decay_rates || d->decay_form == NTK_DECAY_EXP_SOFTPLUS;
+    return d->G > 0 || d->unit_q || d->unit_k || d->head_gates || d->write_gated || d->decay_rates || d->decay_form == NTK_DECAY_EXP_SOFTPLUS || d->conv_w;
 }
 
 static size_t rec_scratch(int T, int H, int dn, int dv, bool removal, bool always, bool values) {
@@ -515,7 +585,7 @@ size_t ntk_gated_recurrence_scratch(int T, int H, int dn, int dv, int removal) {
 
 size_t ntk_gated_recurrence_scratch_ex(const ntk_gated_recurrence_desc* d) {
     if (!d || d->T <= 0 || d->H <= 0 || d->dn <= 0 || d->dv <= 0) return 0;
-    return rec_scratch(d->T, d->H, d->dn, d->dv, d->az != nullptr, rec_needs_prepass(d), d->write_gated != 0);
+    return rec_scratch(d->T, d->H, d->dn, d->dv, d->az != nullptr, rec_needs_prepass(d), d->write_gated != 0 || d->conv_w != nullptr);
 }
 
 int ntk_gated_recurrence(const ntk_gated_recurrence_desc* d, void* stream) {
@@ -526,6 +596,7 @@ int ntk_gated_recurrence(const ntk_gated_recurrence_desc* d, void* stream) {
     if (d->decay_form == NTK_DECAY_SIGMOID_ROOT && !(d->decay_param > 0.0f)) return NTK_E_SHAPE;
     if (d->G < 0 || (d->G > 0 && d->H % d->G)) return NTK_E_SHAPE;
     if (d->write_gated && (!d->az || !d->head_gates)) return NTK_E_SHAPE;   // (the write is scaled by ONE rate per head)
+    if (d->conv_w && (d->T != 1 || d->conv_taps < 1 || d->conv_taps > kStepConvTaps || (d->conv_taps > 1 && !d->conv_state))) return NTK_E_SHAPE;
     const int hd = d->H * d->dn, qd = (d->G > 0 ? d->G : d->H) * d->dn, gd = d->head_gates ? d->H : hd;
     if (d->ldq < qd || d->ldk < qd || d->ldw < gd || (d->az && d->lda < gd) || d->ldv < d->H * d->dv || d->ldo < d->H * d->dv) return NTK_E_SHAPE;
     if (d->T == 0) return NTK_OK;
@@ -533,10 +604,10 @@ int ntk_gated_recurrence(const ntk_gated_recurrence_desc* d, void* stream) {
     if (always && !d->scratch) return NTK_E_NULL;
     RecArgs a{d->out, d->ldo, d->q, d->ldq, d->k, d->ldk, d->v, d->ldv, d->wz, d->ldw, d->wb, d->decay_form, d->decay_param, d->az, d->lda, d->ab, d->unit_eps,
               d->state, d->H, d->dn, d->dv, d->q_scale, d->pos0, d->T, 0, (d->T > kRecFewTokens || always) ? d->scratch : nullptr, 1, d->T, nullptr, nullptr, nullptr, nullptr,
-              d->G, d->unit_q, d->unit_k, d->head_gates, d->write_gated, d->decay_rates, nullptr};
+              d->G, d->unit_q, d->unit_k, d->head_gates, d->write_gated, d->decay_rates, nullptr, d->conv_w, d->conv_state, d->conv_taps};
     if (a.packed) {
         float* next = a.packed + (size_t)d->T * d->H * (d->az ? 5 : 3) * d->dn;
-        if (d->write_gated) { a.vpacked = next; next += (size_t)d->T * d->H * d->dv; }
+        if (d->write_gated || d->conv_w) { a.vpacked = next; next += (size_t)d->T * d->H * d->dv; }
         a.nseg = rec_segments(d->T, d->H, d->dn, d->dv, d->az != nullptr);
         if (a.nseg > 1) {
             a.seg_len = (d->T + a.nseg - 1) / a.nseg;

@@ -55,7 +55,8 @@ class GatedRecurrenceDesc(C.Structure):
                 ("wz", C.c_void_p), ("ldw", C.c_int), ("wb", C.c_void_p), ("decay_form", C.c_int), ("decay_param", C.c_float),
                 ("az", C.c_void_p), ("lda", C.c_int), ("ab", C.c_void_p), ("unit_eps", C.c_float), ("state", C.c_void_p),
                 ("H", C.c_int), ("dn", C.c_int), ("dv", C.c_int), ("q_scale", C.c_float), ("pos0", C.c_int), ("T", C.c_int), ("scratch", C.c_void_p),
-                ("G", C.c_int), ("unit_q", C.c_int), ("unit_k", C.c_int), ("head_gates", C.c_int), ("write_gated", C.c_int), ("decay_rates", C.c_void_p)]
+                ("G", C.c_int), ("unit_q", C.c_int), ("unit_k", C.c_int), ("head_gates", C.c_int), ("write_gated", C.c_int), ("decay_rates", C.c_void_p),
+                ("conv_w", C.c_void_p), ("conv_state", C.c_void_p), ("conv_taps", C.c_int)]
 
 
 DECAY_GIVEN, DECAY_SIGMOID_ROOT, DECAY_EXP_SIGMOID, DECAY_EXP_SOFTPLUS = 0, 1, 2, 3
@@ -517,7 +518,7 @@ def gated_seam(x, y=None, g=None, yb=None, gb=None, hist=None, coef=None, norm=N
 
 def gated_recurrence(q, k, v, wz, H: int, dn: int, dv: int, pos0: int, decay_form: int = DECAY_GIVEN, decay_param: float = 1.0, wb=None, az=None, ab=None,
                      unit_eps: float = 1e-6, q_scale: float = 1.0, state: Optional[np.ndarray] = None, prepass: bool = True, G: int = 0, unit_q: bool = False,
-                     unit_k: bool = False, head_gates: bool = False, write_gated: bool = False, decay_rates=None):
+                     unit_k: bool = False, head_gates: bool = False, write_gated: bool = False, decay_rates=None, conv_w=None, conv_state=None):
     """-> (out [T, H * dv], state [H, dn, dv]); az: the removal rate's raw projection (None: no removal term); state: what an earlier portion left (ignored when
     pos0 == 0; by default full of NaN so that a read at the start would show); prepass: give the scratch that lets longer portions form their per-token vectors
     in a launch of their own"""
@@ -532,11 +533,21 @@ def gated_recurrence(q, k, v, wz, H: int, dn: int, dv: int, pos0: int, decay_for
                             pos0, T, None)
     rb = _f(decay_rates) if decay_rates is not None else None
     d.G, d.unit_q, d.unit_k, d.head_gates, d.write_gated, d.decay_rates = G, int(unit_q), int(unit_k), int(head_gates), int(write_gated), rb.ptr if rb else None
+    cwb = csb = None
+    if conv_w is not None:      # one token whose raw q, k, v pass their short convolutions inside the pre-pass; the carried inputs come back as a third result
+        taps, nch = conv_w.shape[1], conv_w.shape[0]
+        cwb = _f(conv_w)
+        csb = _f(conv_state) if conv_state is not None and np.size(conv_state) else DeviceBuffer.from_numpy(np.full(max(taps - 1, 1) * nch, np.nan, np.float32))
+        d.conv_w, d.conv_state, d.conv_taps = cwb.ptr, csb.ptr, taps
     ns = int(L.ntk_gated_recurrence_scratch_ex(C.byref(d))) if prepass else 0
     scr = DeviceBuffer.from_numpy(np.full(ns, np.nan, np.float32)) if ns else None
     if scr:
         d.scratch = scr.ptr
     check(L.ntk_gated_recurrence(C.byref(d), None), "ntk_gated_recurrence")
+    if csb is not None:
+        taps, nch = conv_w.shape[1], conv_w.shape[0]
+        return (out.numpy(np.float32, T * H * dv).reshape(T, H * dv), sb.numpy(np.float32, H * dn * dv).reshape(H, dn, dv),
+                csb.numpy(np.float32, max(taps - 1, 1) * nch).reshape(max(taps - 1, 1), nch)[:taps - 1])
     return out.numpy(np.float32, T * H * dv).reshape(T, H * dv), sb.numpy(np.float32, H * dn * dv).reshape(H, dn, dv)
 
 

@@ -294,6 +294,34 @@ def test_delta_rule_long_portions_walked_in_segments(H, G, dn, dv):
     assert rel(np.concatenate([a, b]), ref.reshape(T, H * dv)) < 1e-4 and rel(st, S) < 1e-4
 
 
+@pytest.mark.parametrize("H,G,dn,dv,taps", [(4, 2, 8, 8, 4), (6, 3, 32, 64, 4), (3, 3, 13, 7, 2), (2, 1, 70, 130, 5), (5, 1, 16, 300, 1), (2, 2, 128, 96, 16)])
+def test_decoded_tokens_pass_their_convolutions_inside_the_recurrence(H, G, dn, dv, taps):
+    """raw q, k, v of one token at a time, the short convolutions inside the pre-pass's launch: the same outputs, state and carried inputs as the convolution as an
+    operator of its own in front of a whole portion; a sequence may change from one form to the other at any token"""
+    from ntransformer_amd import layers as Lr
+    g = np.random.default_rng(H * 100 + dn + taps)
+    T = 21
+    q, k, v, az, wz, rates, bias = _delta_inputs(g, T, H, G, dn, dv)
+    cw = f32(g.standard_normal((2 * G * dn + H * dv, taps)) * 0.5)
+    raw = np.concatenate([q, k, v], axis=1)
+    conv, carried = O.short_conv(raw.astype(np.float64), cw.astype(np.float64))
+    cq, ck, cv = f32(conv[:, :G * dn]), f32(conv[:, G * dn:2 * G * dn]), f32(conv[:, 2 * G * dn:])
+    ref, S = _delta_reference(cq, ck, cv, az, wz, rates, bias, H, G, dn, dv)
+    kw = dict(decay_form=Lr.DECAY_EXP_SOFTPLUS, wb=bias, decay_rates=rates, G=G, unit_q=True, unit_k=True, head_gates=True, write_gated=True, q_scale=dn ** -0.5)
+    for first in (0, 9):                                                     # the first tokens as one portion through the operators, the rest token by token
+        outs, st, cst = [], None, None
+        if first:
+            conv_a, cst = Lr.causal_conv_act(raw[:first], cw, 0)
+            o, st = Lr.gated_recurrence(conv_a[:, :G * dn], conv_a[:, G * dn:2 * G * dn], conv_a[:, 2 * G * dn:], wz[:first], H, dn, dv, 0, az=az[:first], **kw)
+            outs.append(o)
+        for t in range(first, T):
+            o, st, cst = Lr.gated_recurrence(q[t:t + 1], k[t:t + 1], v[t:t + 1], wz[t:t + 1], H, dn, dv, t, az=az[t:t + 1], state=st, conv_w=cw, conv_state=cst, **kw)
+            outs.append(o)
+        assert rel(np.concatenate(outs), ref.reshape(T, H * dv)) < 1e-5 and rel(st, S) < 1e-5, first
+        if taps > 1:
+            assert np.allclose(cst, carried, atol=1e-6)
+
+
 def test_the_delta_rule_replaces_what_a_key_held_and_remembers_it_without_decay():
     """decay one (a large negative pre-activation), write strength one: a key written at token 0 is read back 600 tokens later; writing the SAME key again
     replaces its value instead of adding to it -- plain linear attention would return the sum"""
