@@ -116,17 +116,31 @@ __global__ __launch_bounds__(64) void gated_recurrence_prepare_kernel(const RecA
 // value channels of the state heads that share them (each channel's carried inputs are read, used and shifted by the one thread that owns the channel), then
 // forms the same vectors as the kernel above, with the same sums in the same lane order.
 constexpr int kStepConvTaps = 16;
-__device__ __forceinline__ float conv_step(const float* w, float* state, int taps, int n, int c, float x, int pos0) {
-    float s = 0.0f;
-    for (int j = 0; j + 1 < taps; ++j) {
-        const float hj = pos0 - (taps - 1) + j >= 0 ? state[(long long)j * n + c] : 0.0f;
-        s = fmaf(w[(long long)c * taps + j], hj, s);
-        if (j > 0) state[(long long)(j - 1) * n + c] = hj;
+struct ConvTaps {                                        // one channel's carried inputs, taps and present input, all requested before anything is stored
+    float hist[kStepConvTaps - 1], w[kStepConvTaps], x;
+    __device__ __forceinline__ void load(const float* cw, const float* state, int taps, int n, int c, float xin, int pos0) {
+#pragma unroll
+        for (int j = 0; j < kStepConvTaps - 1; ++j) hist[j] = (j < taps - 1 && pos0 - (taps - 1) + j >= 0) ? state[(long long)j * n + c] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < kStepConvTaps; ++j) w[j] = j < taps ? cw[(long long)c * taps + j] : 0.0f;
+        x = xin;
     }
-    s = fmaf(w[(long long)c * taps + taps - 1], x, s);
-    if (taps > 1) state[(long long)(taps - 2) * n + c] = x;
-    return s / (1.0f + expf(-s));
-}
+    // the convolution and silu; the carried rows shift in place
+    __device__ __forceinline__ float finish(float* state, int taps, int n, int c) const {
+        float s = 0.0f;
+#pragma unroll
+        for (int j = 0; j < kStepConvTaps - 1; ++j)
+            if (j < taps - 1) s = fmaf(w[j], hist[j], s);
+#pragma unroll
+        for (int j = 0; j < kStepConvTaps; ++j)
+            if (j == taps - 1) s = fmaf(w[j], x, s);
+#pragma unroll
+        for (int j = 1; j < kStepConvTaps - 1; ++j)
+            if (j < taps - 1) state[(long long)(j - 1) * n + c] = hist[j];
+        if (taps > 1) state[(long long)(taps - 2) * n + c] = x;
+        return s / (1.0f + expf(-s));
+    }
+};
 
 template <bool DELTA>
 __global__ __launch_bounds__(256) void gated_recurrence_prepare_step_kernel(const RecArgs a) {
@@ -137,9 +151,32 @@ __global__ __launch_bounds__(256) void gated_recurrence_prepare_step_kernel(cons
     const int nch = 2 * G * a.dn + a.H * a.dv;           // convolved channels: q | k | v
     float* qs = cs;
     float* ks = cs + a.dn;
-    for (int d = threadIdx.x; d < a.dn; d += 256) {
-        qs[d] = conv_step(a.conv_w, a.conv_state, a.conv_taps, nch, g * a.dn + d, a.q[(long long)g * a.dn + d], a.pos0);
-        ks[d] = conv_step(a.conv_w, a.conv_state, a.conv_taps, nch, G * a.dn + g * a.dn + d, a.k[(long long)g * a.dn + d], a.pos0);
+    // the gates of the wave's first state head: requested now, used after the convolutions
+    float wz0 = 0.0f, az0 = 0.0f, rate0 = a.decay_param;
+    if (a.head_gates && wave < R) {
+        const int h = g * R + wave;
+        wz0 = a.wz[h] + (a.wb ? a.wb[h] : 0.0f);
+        if (a.decay_rates) rate0 = a.decay_rates[h];
+        if constexpr (DELTA) az0 = a.az[h] + (a.ab ? a.ab[h] : 0.0f);
+    }
+    const int nqk = 2 * a.dn, nv = R * a.dv;
+    for (int e = threadIdx.x; e < max(nqk, nv); e += 256) {
+        // the head's q and k channels, and the value channels of the state heads that share them (times the head's removal rate): one round of requests for both
+        ConvTaps A, B;
+        const bool ha = e < nqk, hb = e < nv;
+        const int which = e / a.dn, d = e % a.dn, cA = which * G * a.dn + g * a.dn + d;
+        const int h = g * R + e / a.dv, c = e % a.dv, cB = 2 * G * a.dn + h * a.dv + c;
+        float azv = 0.0f;
+        if (ha) A.load(a.conv_w, a.conv_state, a.conv_taps, nch, cA, which ? a.k[(long long)g * a.dn + d] : a.q[(long long)g * a.dn + d], a.pos0);
+        if (hb) {
+            B.load(a.conv_w, a.conv_state, a.conv_taps, nch, cB, a.v[(long long)h * a.dv + c], a.pos0);
+            if constexpr (DELTA) { if (a.write_gated) azv = a.az[h] + (a.ab ? a.ab[h] : 0.0f); }
+        }
+        if (ha) cs[e] = A.finish(a.conv_state, a.conv_taps, nch, cA);
+        if (hb) {
+            const float vv = B.finish(a.conv_state, a.conv_taps, nch, cB);
+            a.vpacked[(long long)h * a.dv + c] = (DELTA && a.write_gated) ? vv * (1.0f / (1.0f + expf(-azv))) : vv;
+        }
     }
     __syncthreads();
     float ss = 0.0f, sq = 0.0f;
@@ -153,8 +190,9 @@ __global__ __launch_bounds__(256) void gated_recurrence_prepare_step_kernel(cons
         const long long oc = (long long)h * a.dn;
         float wh = 1.0f, ah = 0.0f;
         if (a.head_gates) {
-            wh = decay_of(a.wz[h] + (a.wb ? a.wb[h] : 0.0f), a.decay_form, a.decay_rates ? a.decay_rates[h] : a.decay_param);
-            if constexpr (DELTA) ah = 1.0f / (1.0f + expf(-(a.az[h] + (a.ab ? a.ab[h] : 0.0f))));
+            const bool first = r == wave;
+            wh = decay_of(first ? wz0 : a.wz[h] + (a.wb ? a.wb[h] : 0.0f), a.decay_form, first ? rate0 : a.decay_rates ? a.decay_rates[h] : a.decay_param);
+            if constexpr (DELTA) ah = 1.0f / (1.0f + expf(-(first ? az0 : a.az[h] + (a.ab ? a.ab[h] : 0.0f))));
         }
         for (int d = lane; d < a.dn; d += 64) {
             const float kk = ks[d];
@@ -168,10 +206,6 @@ __global__ __launch_bounds__(256) void gated_recurrence_prepare_step_kernel(cons
                 dst[3 * a.dn + d] = a.write_gated ? uu * w : uu;
                 dst[4 * a.dn + d] = uu * aa;
             }
-        }
-        for (int c = lane; c < a.dv; c += 64) {
-            const float vv = conv_step(a.conv_w, a.conv_state, a.conv_taps, nch, 2 * G * a.dn + h * a.dv + c, a.v[(long long)h * a.dv + c], a.pos0);
-            a.vpacked[(long long)h * a.dv + c] = (DELTA && a.write_gated) ? vv * ah : vv;
         }
     }
 }
