@@ -190,7 +190,7 @@ def fifotar_config(preset: str, layers: int = 4, mlp_everywhere: bool = True) ->
     ls = []
     for k in range(layers):
         if k % 4 == 0:
-            mx = {"heads": H, "kv_heads": max(H // 4, 1), "dim": dn, "vdim": dv, "scale": 1.0 / math.sqrt(dn), "softcap": 50.0, "mask": {"size": p["window"]}, "v_mix": True}
+            mx = {"heads": H, "kv_heads": max(H // 4, 1), "dim": dn, "vdim": dv, "scale": 1.0 / math.sqrt(dn), "softcap": 40.0, "mask": {"size": p["window"]}, "v_mix": True}
             t = "attention"
         elif k % 4 == 2:
             mx = {"heads": H, "dim": dn, "rot_dim": p["rot_dim"], "vdim": dv, "kv_rank": p["kv_rank"], "q_rank": p["q_rank"], "scale": 1.0 / math.sqrt(dn + p["rot_dim"]),
@@ -201,7 +201,7 @@ def fifotar_config(preset: str, layers: int = 4, mlp_everywhere: bool = True) ->
             t = "delta"
         has_mlp = mlp_everywhere or t != "delta"
         ls.append({"type": t, "mixer": mx, "mlp": {"kind": "dense", "ff": max(ff, 64), "limit": 7.0} if has_mlp else None})
-    return {"architecture": "Fifotar", "layers": ls, "norm": {"eps": 1e-5}, "embedding": {"scale": math.sqrt(p["width"])}, "residual_mult": 0.5, "logit_softcap": 30.0,
+    return {"architecture": "Fifotar", "layers": ls, "norm": {"eps": 1e-5}, "embedding": {"scale": math.sqrt(p["width"])}, "residual_mult": 0.7, "logit_softcap": 25.0,
             "vocab": p["vocab"], "width": p["width"]}
 
 

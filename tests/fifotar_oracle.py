@@ -293,7 +293,7 @@ def delta_layer(heads=4, kv_heads=2, dim=8, vdim=8, conv=4, ff=0, limit=2.0):
     return {"type": "delta", "mixer": mx, "mlp": {"kind": "dense", "ff": ff, "limit": limit} if ff else None}
 
 
-def config(layers, vocab=61, width=32, eps=1e-5, mult=0.5, embed_scale=None, logit_softcap=30.0):
+def config(layers, vocab=61, width=32, eps=1e-5, mult=0.6, embed_scale=None, logit_softcap=25.0):
     cfg = {"architecture": "Fifotar", "vocab": vocab, "width": width, "norm": {"eps": eps}, "residual_mult": mult,
            "embedding": {"scale": embed_scale if embed_scale is not None else math.sqrt(width)}, "layers": layers}
     if logit_softcap:

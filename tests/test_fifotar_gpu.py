@@ -115,7 +115,7 @@ def test_logit_cap_and_gate_per_head():
     assert rel(Lr.latent_unfold_value(lat, wuv, 3, gate=gt[:4], head_gate=True), ref.reshape(4, 15)) < 1e-6
 
 
-@pytest.mark.parametrize("scaling", [None, {"factor": 4.0, "original": 16, "fast": 4.0, "slow": 1.0}, {"factor": 2.0, "original": 512, "fast": 32.0, "slow": 1.0}])
+@pytest.mark.parametrize("scaling", [None, {"factor": 4.0, "original": 16, "fast": 4.0, "slow": 1.0}, {"factor": 3.0, "original": 256, "fast": 16.0, "slow": 2.0}])
 def test_half_split_rotation_into_cache_rows_and_queries(scaling):
     from ntransformer_amd import layers as Lr
     g = np.random.default_rng(5)
@@ -502,7 +502,7 @@ def test_other_sizes(tmp_path, name):
 def test_long_decoding_and_a_prompt_longer_than_one_internal_pass(tmp_path):
     """1100 tokens are two internal passes: the blended values are those of each pass's own tokens, the convolutions and the state carry across; then 200 tokens
     one by one across several chunk edges"""
-    cfg = O.config([O.attention_layer(size=96), O.delta_layer(), O.attention_layer(size=200), O.latent_layer(ff=0)])
+    cfg = O.config([O.attention_layer(size=88), O.delta_layer(), O.attention_layer(size=200), O.latent_layer(ff=0)])
     folder, w = make(tmp_path, cfg, seed=9)
     toks = tokens_for(cfg, 1100, seed=10)
     e = engine_for(folder, ctx=1300)
