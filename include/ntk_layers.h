@@ -229,6 +229,9 @@ typedef struct ntk_window_attention_desc {
      * softcap > 0: the scaled (and biased) score s becomes softcap * tanh(s / softcap).
      * sink != 0: one more term exp(0) in the softmax's denominator (a key of score 0 that carries no value): p_j = exp(s_j) / (1 + sum exp(s)). */
     int mask_mode; float softcap; int sink;
+    /* gate != NULL: the result (after the pair, the unit norm and out_scale) times sigmoid(gate[t][h][c]), gate rows ldg floats apart: an elementwise output gate
+     * inside the launch that writes the result */
+    const float* gate; int ldg;
 } ntk_window_attention_desc;
 #define NTK_MASK_SLIDING 0
 #define NTK_MASK_CHUNKS 1

@@ -950,8 +950,8 @@ int LayerStackModel::run_window(const StackLayer& L, float* cache, int T, int po
     d.sub_norm = m.maps == 2 ? 1 : 0; d.eps = eps_; d.out_scale = m.maps == 2 ? 1.0f - m.diff : 1.0f;
     d.scratch = wscratch_;
     d.mask_mode = m.mask_mode; d.softcap = m.softcap; d.sink = m.sink ? 1 : 0;
+    if (m.gated) { d.gate = a_ + m.g_off; d.ldg = na; }     // the elementwise gate rides in the launch that writes the heads' results
     LS_TRY(ntk_window_attention(&d, stream_));
-    if (m.gated) LS_TRY(ntk_sigmoid_gate(att_, hv, a_ + m.g_off, na, T, hv, stream_));
     return ntk_dense_linear(mix_, W, att_, hv, m.o.ptr, m.o.dtype, T, W, hv, 0, stream_);
 }
 

@@ -78,6 +78,7 @@ struct WinArgs {
     int splits; float* scratch;       // splits > 1: states [T * H][splits][maps][2 + dv]
     const float* rel; const int* bucket_of; int n_dist;   // rel != NULL: rel[bucket_of[min(distance, n_dist - 1)] * H + head] joins the scaled score
     int chunks; float softcap; int sink;                  // chunks != 0: `window` is a chunk size
+    const float* gate; int ldg;                           // gate != NULL: out[t][h][c] *= sigmoid(gate[t * ldg + h * dv + c])
 };
 
 // first key a query at position p sees
@@ -90,7 +91,7 @@ constexpr int WROWS = 16, WQPW = 4, WKCH = 64, WSLAB = 64, WMAXC = 8;   // dv <=
 
 // the differential pair, the unit norm and the scale on a row whose lanes hold columns c * 64 + lane
 template <int M>
-__device__ __forceinline__ void finish_row(float (&a)[M][WMAXC], int lane, int dv, float lambda, int sub_norm, float eps, float out_scale, float* o) {
+__device__ __forceinline__ void finish_row(float (&a)[M][WMAXC], int lane, int dv, float lambda, int sub_norm, float eps, float out_scale, float* o, const float* gate) {
     float r[WMAXC];
     float ss = 0.0f;
 #pragma unroll
@@ -105,7 +106,7 @@ __device__ __forceinline__ void finish_row(float (&a)[M][WMAXC], int lane, int d
     if (sub_norm) mul = out_scale / sqrtf(wave_sum(ss) / (float)dv + eps);
 #pragma unroll
     for (int c = 0; c < WMAXC; ++c)
-        if (c * WSLAB + lane < dv) o[c * WSLAB + lane] = r[c] * mul;
+        if (c * WSLAB + lane < dv) o[c * WSLAB + lane] = gate ? r[c] * mul / (1.0f + expf(-gate[c * WSLAB + lane])) : r[c] * mul;
 }
 
 template <int M>
@@ -263,7 +264,8 @@ __global__ __launch_bounds__(256) void window_attention_kernel(const WinArgs a) 
 #pragma unroll
             for (int c = 0; c < WMAXC; ++c) r[m][c] = acc[m][i][c] * inv;
         }
-        finish_row<M>(r, lane, a.dv, a.lambda, a.sub_norm, a.eps, a.out_scale, a.out + (long long)t * a.ldo + (long long)h * a.dv);
+        finish_row<M>(r, lane, a.dv, a.lambda, a.sub_norm, a.eps, a.out_scale, a.out + (long long)t * a.ldo + (long long)h * a.dv,
+                      a.gate ? a.gate + (long long)t * a.ldg + (long long)h * a.dv : nullptr);
     }
 }
 
@@ -303,7 +305,8 @@ __global__ __launch_bounds__(64) void window_attention_merge_kernel(const WinArg
 #pragma unroll
         for (int c = 0; c < WMAXC; ++c) r[m][c] *= inv;
     }
-    finish_row<M>(r, lane, a.dv, a.lambda, a.sub_norm, a.eps, a.out_scale, a.out + (long long)(row / a.H) * a.ldo + (long long)(row % a.H) * a.dv);
+    finish_row<M>(r, lane, a.dv, a.lambda, a.sub_norm, a.eps, a.out_scale, a.out + (long long)(row / a.H) * a.ldo + (long long)(row % a.H) * a.dv,
+                  a.gate ? a.gate + (long long)(row / a.H) * a.ldg + (long long)(row % a.H) * a.dv : nullptr);
 }
 
 // parts the key chunks of a row tile go round: only when few tiles face many chunks
@@ -373,6 +376,8 @@ int ntk_window_attention(const ntk_window_attention_desc* d, void* stream) {
     a.pos0 = d->pos0; a.T = d->T; a.window = d->window; a.scale = d->scale; a.lambda = d->lambda; a.sub_norm = d->sub_norm; a.eps = d->eps; a.out_scale = d->out_scale;
     if ((d->mask_mode != NTK_MASK_SLIDING && d->mask_mode != NTK_MASK_CHUNKS) || d->softcap < 0.0f) return NTK_E_SHAPE;
     a.chunks = d->mask_mode == NTK_MASK_CHUNKS; a.softcap = d->softcap; a.sink = d->sink;
+    if (d->gate && d->ldg < d->H * d->dv) return NTK_E_SHAPE;
+    a.gate = d->gate; a.ldg = d->ldg;
     a.splits = d->scratch ? window_splits(d->T, d->H, d->G, window_keys(d->pos0, d->T, d->window, a.chunks)) : 1;
     a.scratch = d->scratch;
     a.rel = d->rel; a.bucket_of = d->bucket_of; a.n_dist = d->n_dist;

@@ -41,7 +41,8 @@ class WindowAttentionDesc(C.Structure):
     _fields_ = [("out", C.c_void_p), ("ldo", C.c_int), ("q", C.c_void_p), ("ldq", C.c_int), ("cache", C.c_void_p), ("row", C.c_int),
                 ("H", C.c_int), ("G", C.c_int), ("maps", C.c_int), ("dn", C.c_int), ("dv", C.c_int), ("pos0", C.c_int), ("T", C.c_int), ("window", C.c_int),
                 ("scale", C.c_float), ("lam", C.c_float), ("sub_norm", C.c_int), ("eps", C.c_float), ("out_scale", C.c_float), ("scratch", C.c_void_p),
-                ("rel", C.c_void_p), ("bucket_of", C.c_void_p), ("n_dist", C.c_int), ("mask_mode", C.c_int), ("softcap", C.c_float), ("sink", C.c_int)]
+                ("rel", C.c_void_p), ("bucket_of", C.c_void_p), ("n_dist", C.c_int), ("mask_mode", C.c_int), ("softcap", C.c_float), ("sink", C.c_int),
+                ("gate", C.c_void_p), ("ldg", C.c_int)]
 
 
 class GatedSeamDesc(C.Structure):
@@ -387,7 +388,7 @@ def window_prepare_biased(q, k, v, H: int, G: int, dn: int, dv: int, pos0: int, 
 
 def window_attention(q: np.ndarray, cache: np.ndarray, H: int, G: int, maps: int, dn: int, dv: int, pos0: int, window: int, scale: float, lam: float = 0.0,
                      sub_norm: bool = False, eps: float = 1e-6, out_scale: float = 1.0, split: bool = True, rel: Optional[np.ndarray] = None,
-                     bucket_of: Optional[np.ndarray] = None, chunks: bool = False, softcap: float = 0.0, sink: bool = False) -> np.ndarray:
+                     bucket_of: Optional[np.ndarray] = None, chunks: bool = False, softcap: float = 0.0, sink: bool = False, gate: Optional[np.ndarray] = None) -> np.ndarray:
     """q [T, H * maps * dn] (rotated), cache rows [G][maps][dn] keys | [G][dv] values; split: long key ranges of few rows may be cut into merged parts;
     rel [buckets, H] with bucket_of [distances]: a bias by distance on the scaled score"""
     L = _bind()
@@ -401,6 +402,9 @@ def window_attention(q: np.ndarray, cache: np.ndarray, H: int, G: int, maps: int
         rb, bb = _f(rel), _i(bucket_of)
         d.rel, d.bucket_of, d.n_dist = rb.ptr, bb.ptr, len(bucket_of)
     d.mask_mode, d.softcap, d.sink = (MASK_CHUNKS if chunks else MASK_SLIDING), softcap, int(sink)
+    if gate is not None:        # [T, H * dv]: an elementwise sigmoid gate on the result
+        gb = _f(gate)
+        d.gate, d.ldg = gb.ptr, gate.shape[1]
     check(L.ntk_window_attention(C.byref(d), None), "ntk_window_attention")
     return out.numpy(np.float32, T * H * dv).reshape(T, H * dv)
 

@@ -172,9 +172,12 @@ def test_attention_over_chunks_with_capped_scores_and_a_sink(H, G, dn, dv, pos0,
     scale = 2.0 / math.sqrt(dn)
     ref = O.attend(q[pos0:].reshape(T, H, dn).astype(np.float64), K.reshape(P, G, dn).astype(np.float64), V.reshape(P, G, dv).astype(np.float64), pos0, scale,
                    size or None, cap or None, sink).reshape(T, H * dv)
+    gate = f32(g.standard_normal((T, H * dv)) * 2)
     for split in (True, False):
         got = Lr.window_attention(q[pos0:], cache, H, G, 1, dn, dv, pos0, size, scale, split=split, chunks=True, softcap=cap, sink=sink)
         assert rel(got, ref) < 1e-5, split
+        got = Lr.window_attention(q[pos0:], cache, H, G, 1, dn, dv, pos0, size, scale, split=split, chunks=True, softcap=cap, sink=sink, gate=gate)   # the gate inside the launch
+        assert rel(got, ref * O.sigmoid(gate.astype(np.float64))) < 1e-5, split
 
 
 def test_the_sink_takes_the_weight_when_every_score_is_low():
