@@ -284,7 +284,7 @@ typedef struct ntk_gated_recurrence_desc {
      * unit_q / unit_k != 0: q (before q_scale) / the written key k are divided by sqrt(sum x^2 + unit_eps) over the head's dn entries.
      * head_gates != 0: wz and az hold ONE number per token and head ([T][H], ldw / lda >= H; wb, ab [H]): a decay and a removal rate for all channels.
      * decay_form NTK_DECAY_EXP_SOFTPLUS: w = exp(-rate * softplus(z)), rate = decay_rates[h] (device F32 [H]) or decay_param where that is NULL.
-     * write_gated != 0 (needs az): the delta rule proper -- the removal is taken from the DECAYED state and the write is scaled by the removal rate:
+     * write_gated != 0 (needs az and head_gates): the delta rule proper -- the removal is taken from the DECAYED state and the write is scaled by the removal rate:
      *     S' = diag(w_t) S_(t-1),   S_t = S' - a_t u_t (u_t^T S') + a_t k_t v_t^T
      * Any of these makes every portion form its vectors in a launch of its own: scratch must hold ntk_gated_recurrence_scratch_ex(d) floats. */
     int G, unit_q, unit_k, head_gates, write_gated;

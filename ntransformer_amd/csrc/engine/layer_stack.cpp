@@ -794,8 +794,9 @@ int LayerStackModel::alloc_buffers() {
             max_in_ = std::max<int>(max_in_, (int)m.in.out_f);
             max_hdv_ = std::max(max_hdv_, m.heads * m.vdim);
             max_conv_ = std::max(max_conv_, m.channels());
+            static const float removal = 0.0f;         // (the size only asks whether there is a removal term)
             ntk_gated_recurrence_desc d{};
-            d.T = chunk_; d.H = m.heads; d.dn = m.dim; d.dv = m.vdim; d.az = (const float*)&d; d.head_gates = 1; d.write_gated = 1;   // (az: only whether there is a removal term is looked at)
+            d.T = chunk_; d.H = m.heads; d.dn = m.dim; d.dv = m.vdim; d.az = &removal; d.head_gates = 1; d.write_gated = 1;
             rsc = std::max(rsc, ntk_gated_recurrence_scratch_ex(&d));
         } else if (L.mixer == kMixWindow) {
             const WindowMixer& m = L.att;
